@@ -189,9 +189,32 @@ pegainfer_status_t pegainfer_route_topk(const void* h, const void* w_router, con
 pegainfer_status_t pegainfer_route_from_logits(const float* logits, const void* correction, int32_t* out_expert, float* out_weight,
                                                int32_t experts, int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
                                                int32_t score_kind, int32_t dtype, pegainfer_stream_t stream);
+/* the same with the logits at a row stride of their own (a GEMM may leave other columns beside them), a choice of the group
+ * score (the sum of a group's two largest choices, or its largest) and, with renorm != 0, weights divided by their sum + 1e-20 */
+enum { PEGAINFER_GROUP_TOP2_SUM = 0, PEGAINFER_GROUP_MAX = 1 };
+pegainfer_status_t pegainfer_route_from_logits_ex(const float* logits, int64_t logits_stride, const void* correction,
+                                                  int32_t* out_expert, float* out_weight, int32_t experts, int32_t n_groups,
+                                                  int32_t keep_groups, int32_t top, int32_t rows, int32_t score_kind,
+                                                  int32_t group_kind, int32_t renorm, int32_t dtype, pegainfer_stream_t stream);
 /* pegainfer_route_combine plus a row every token gets (a shared expert's output, [rows, d] of dtype; NULL = none) */
 pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float* weight, const void* add, void* out, int32_t d,
                                                int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream);
+
+/* pegainfer_route_combine_add whose added row is first multiplied by sigmoid(add_gate[row * add_gate_stride]) (fp32 logits, one
+ * per row; NULL = no gate) */
+pegainfer_status_t pegainfer_route_combine_gated(const float* y_pairs, const float* weight, const void* add,
+                                                 const float* add_gate, int64_t add_gate_stride, void* out, int32_t d,
+                                                 int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream);
+
+/* Residual sum with a constant factor, then an RMS norm whose gain is ONE number (gain: a one-element tensor of dtype):
+ *   r = x_in + mult * (y + bias) + add_rows + add_vec          -> x_out (fp32; may alias x_in)
+ *   n = r / sqrt(mean(r^2) + eps) * gain[0]                    -> n_out (fp32)
+ * y [rows, d] of y_dtype or NULL (then bias and mult are unused); bias, add_vec [d] of dtype or NULL; add_rows fp32 [rows, d] or
+ * NULL; x_out or n_out may be NULL. */
+pegainfer_status_t pegainfer_scalar_rms_add(const float* x_in, const void* y, int32_t y_dtype, const void* bias, float mult,
+                                            const float* add_rows, const void* add_vec, float* x_out, const void* gain,
+                                            float eps, float* n_out, int32_t d, int32_t rows, int32_t dtype,
+                                            pegainfer_stream_t stream);
 
 /* ---- recurrent matrix memories (state per (slot, head): S [dim][vdim] fp32, row-major) ----
  * Gated delta rule.  Per row, from qkv (fp32 [rows][qkv_stride]: q heads at 0, k heads at kv_heads * dim, v heads at
@@ -205,6 +228,16 @@ pegainfer_status_t pegainfer_delta_rule(float* qkv, int64_t qkv_stride, const vo
                                         int64_t slot_stride, float* o, int32_t heads, int32_t kv_heads, int32_t dim,
                                         int32_t vdim, int32_t n_rows, const int32_t* entry_row0, const int32_t* entry_slot,
                                         int32_t n_entries, int32_t dtype, pegainfer_stream_t stream);
+/* The gated delta rule with one decay per (head, key channel), acting on the rows of S:  g = exp(-exp(A_log[h]) *
+ * softplus(a[row, h * dim + d] + dt_bias[h * dim + d])), a: fp32 [rows][heads * dim] at stride a_stride (the output of the decay
+ * projection), dt_bias [heads * dim], A_log [heads]; gates: fp32 scratch [rows][heads * dim + heads].  Everything else as
+ * pegainfer_delta_rule. */
+pegainfer_status_t pegainfer_delta_rule_channel(float* qkv, int64_t qkv_stride, const void* proj, int64_t proj_stride,
+                                                int64_t b_off, const float* a, int64_t a_stride, const void* A_log,
+                                                const void* dt_bias, float* gates, float* state, int64_t slot_stride, float* o,
+                                                int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t n_rows,
+                                                const int32_t* entry_row0, const int32_t* entry_slot, int32_t n_entries,
+                                                int32_t dtype, pegainfer_stream_t stream);
 /* Exponentially gated matrix memory with a running maximum (state per (slot, head): S [dim][vdim], n [dim], m; the slot's
  * region is [S of all heads | n of all heads | m of all heads]).  Per row from `proj` (dtype): q at q_off, k at k_off
  * (heads x dim), v at v_off (heads x vdim), gate inputs at i_off / f_off (one per head), biases i_bias / f_bias:
@@ -242,6 +275,17 @@ pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_s
                                                 int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
                                                 int32_t page_size, float* q_out, void* q_out_stored, int32_t n_rows,
                                                 int32_t dtype, pegainfer_stream_t stream);
+/* The same with more options: q_norm / k_norm may both be NULL (no norm); q_bias [heads * dim], k_bias [kv_heads * dim],
+ * v_bias [kv_heads * vdim] of dtype or NULL are added to the projection's values first; qt_every > 0 multiplies the query by
+ * 1 + qt_coef * ln(floor((position + 1) / qt_every) + 1) (query temperature); rot_dims may be 0. */
+pegainfer_status_t pegainfer_qk_prep_paged(const void* proj, int64_t proj_stride, int64_t q_off, int64_t k_off, int64_t v_off,
+                                          int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, const void* q_norm,
+                                          const void* k_norm, float eps, const void* q_bias, const void* k_bias,
+                                          const void* v_bias, float qt_coef, int32_t qt_every, const float* inv_freq,
+                                          int32_t rot_dims, const int32_t* positions, const int32_t* row_entry,
+                                          const int32_t* page_indptr, const int32_t* page_ids, void* cache, int64_t page_stride,
+                                          int64_t k_cache_off, int64_t v_cache_off, int32_t page_size, float* q_out,
+                                          void* q_out_stored, int32_t n_rows, int32_t dtype, pegainfer_stream_t stream);
 /* Causal softmax attention, scores and weights in fp32:  out[row, h, :] = factor * sum_{j <= position} softmax_j(q . k_j * scale) v_j.
  * The rows are cut by the caller into tiles that stay inside one entry: tile i covers rows tile_row0[i] .. + tile_ntok[i] - 1
  * and, of each key/value group's query heads, tile_qh0[i] .. + tile_nqh[i] - 1, with ntok * nqh <= 16.  dim, vdim <= 256.
@@ -253,6 +297,19 @@ pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, 
                                              float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
                                              const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
                                              int64_t out_stride, int32_t dtype, pegainfer_stream_t stream);
+/* The same kernel with its options.  maps = 2: a query head and a key head hold [map 1 : dim | map 2 : dim] (q rows and cache
+ * keys are 2 * dim wide), each map is a softmax of its own over the same values, out = map 1 - lambda * map 2 (maps * dim <= 256).
+ * block > 0: a key j is visible to position i only if j <= i and floor(j / block) == floor(i / block), blocks counted from
+ * position 0 of the sequence.  sink: [heads] logits of dtype (or NULL) that join every softmax denominator as exp(sink), without
+ * scale, key or value.  head_norm != 0: out / sqrt(mean(out^2) + norm_eps) over the head's vdim values.  `factor` comes last. */
+pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
+                                                int64_t v_cache_off, int32_t page_size, const int32_t* positions,
+                                                const int32_t* row_entry, const int32_t* page_indptr, const int32_t* page_ids,
+                                                int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float scale,
+                                                float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
+                                                const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
+                                                int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
+                                                int32_t head_norm, float norm_eps, int32_t dtype, pegainfer_stream_t stream);
 /* out[row, :cols] = in[row, :cols] * factor; rows of in / out at their own strides (elements of dtype) */
 pegainfer_status_t pegainfer_scale_rows(const void* in, int64_t in_stride, void* out, int64_t out_stride, int32_t cols,
                                         int32_t rows, float factor, int32_t dtype, pegainfer_stream_t stream);

@@ -1,12 +1,16 @@
 // Softmax attention over a paged key/value cache for any head sizes and grouped key/value heads, in a bf16 and an fp32
 // storage instance; norms, angles, scores, softmax state and accumulators are fp32 in both.
-//   qk_norm_rope_paged_kernel  one workgroup per token row, a wave per head: RMS norm over the head (plain weight), rotation
+//   qk_norm_rope_paged_kernel  one workgroup per token row, a wave per head: optional bias, optional RMS norm over the head
+//                              (plain weight), optional position-dependent query factor (query temperature), rotation
 //                              of neighbouring pairs (2i, 2i + 1) of the first rot_dims values by position * inv_freq[i],
 //                              queries to an fp32 buffer, keys and values into the cache entry of (request, position)
 //   paged_attention_kernel     one workgroup per (row tile, key/value head): up to 16 (token, query head) rows that share the
 //                              key/value head; key and value tiles of 64 positions are staged once in LDS (fp32) for all
 //                              rows; a wave owns up to four rows, a lane one key of the tile for the scores and value
-//                              columns lane, lane + 64, ... for the output; running maximum / sum per row
+//                              columns lane, lane + 64, ... for the output; running maximum / sum per row.  Options
+//                              (AttnForm): keys restricted to the query's own run of `block` positions, a per-head sink
+//                              logit in the denominator, two softmax maps over the same values combined as
+//                              map 1 - lambda * map 2, an RMS norm of the head's output
 // Keys are always visited in tiles of 64 from position 0, whatever the step's shape, so a row's arithmetic does not depend on
 // how its prompt was cut or on what else runs in the step.
 #include <algorithm>
@@ -23,7 +27,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_paged_kernel(
     const A* __restrict__ q_norm, const A* __restrict__ k_norm, float eps, const float* __restrict__ inv_freq, int rot_dims,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_entry, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ page_ids, A* __restrict__ cache, int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
-    int page_size, float* __restrict__ q_out, A* __restrict__ q_out_stored) {
+    int page_size, float* __restrict__ q_out, A* __restrict__ q_out_stored, const A* __restrict__ q_bias,
+    const A* __restrict__ k_bias, const A* __restrict__ v_bias, float qt_coef, int qt_every) {
   extern __shared__ float sm[];   // [4 waves][dim]
   const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pos = positions[row], e = row_entry[row];
@@ -31,19 +36,26 @@ __global__ __launch_bounds__(256) void qk_norm_rope_paged_kernel(
   const int slot = pos % page_size;
   const A* pr = proj + (int64_t)row * proj_stride;
   float* buf = sm + wave * dim;
+  // query temperature: a factor on the whole query that grows with the logarithm of the position's block number
+  const float qt = qt_every > 0 ? 1.0f + qt_coef * logf((float)((pos + 1) / qt_every) + 1.0f) : 1.0f;
   for (int hh = wave; hh < H + G; hh += 4) {
     const bool is_q = hh < H;
     const A* src = is_q ? pr + q_off + (int64_t)hh * dim : pr + k_off + (int64_t)(hh - H) * dim;
     const A* nw = is_q ? q_norm : k_norm;
+    const A* bs = is_q ? (q_bias ? q_bias + (int64_t)hh * dim : nullptr) : (k_bias ? k_bias + (int64_t)(hh - H) * dim : nullptr);
     float ss = 0.f;
     for (int i = lane; i < dim; i += 64) {
-      const float v = ld(src + i);
+      const float v = ld(src + i) + (bs ? ld(bs + i) : 0.f);
       buf[i] = v;
       ss = fmaf(v, v, ss);
     }
-    ss = wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
-    for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * ld(nw + i);
+    if (nw) {
+      ss = wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+      for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * ld(nw + i);
+    }
+    if (is_q && qt_every > 0)
+      for (int i = lane; i < dim; i += 64) buf[i] *= qt;
     __builtin_amdgcn_wave_barrier();
     for (int i = lane; i < dim; i += 64) {
       float out = buf[i];
@@ -60,27 +72,43 @@ __global__ __launch_bounds__(256) void qk_norm_rope_paged_kernel(
     }
     __builtin_amdgcn_wave_barrier();
   }
-  for (int i = threadIdx.x; i < G * vdim; i += 256)
-    cache[page * page_stride + v_cache_off + (int64_t)slot * G * vdim + i] = pr[v_off + i];
+  for (int i = threadIdx.x; i < G * vdim; i += 256) {
+    A* dst = cache + page * page_stride + v_cache_off + (int64_t)slot * G * vdim + i;
+    if (v_bias) st(dst, ld(pr + v_off + i) + ld(v_bias + i));
+    else *dst = pr[v_off + i];
+  }
 }
 
 constexpr int kAttKeys = 64;    // keys per staged tile
 constexpr int kAttRows = 16;    // (token, query head) rows per workgroup
 constexpr int kAttRpw = 4;      // rows per wave
 
-template <typename A>
+// What the general kernel can do beyond plain causal softmax attention; a zeroed struct is the plain form.
+struct AttnForm {
+  int block = 0;               // > 0: a key is visible only inside the query's own run of `block` positions (runs counted from
+                               // position 0 of the sequence), and not after the query
+  const void* sink = nullptr;  // [heads] logits (storage type) that join the softmax denominator, unscaled, without a value
+  float lambda = 0.f;          // MAPS == 2: out = map 1 - lambda * map 2 (two softmax maps over the same values; a query /
+                               // key head holds [map 1 : dim | map 2 : dim])
+  int head_norm = 0;           // != 0: out / sqrt(mean(out^2) + norm_eps) over the head's vdim values, before `factor`
+  float norm_eps = 0.f;
+};
+
+template <typename A, int MAPS>
 __global__ __launch_bounds__(256) void paged_attention_kernel(
     const float* __restrict__ q, const A* __restrict__ cache, int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
     int page_size, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_entry,
     const int32_t* __restrict__ page_indptr, const int32_t* __restrict__ page_ids, int H, int G, int dim, int vdim, float scale,
     float factor, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ tile_ntok,
-    const int32_t* __restrict__ tile_qh0, const int32_t* __restrict__ tile_nqh, A* __restrict__ out, int64_t out_stride) {
+    const int32_t* __restrict__ tile_qh0, const int32_t* __restrict__ tile_nqh, A* __restrict__ out, int64_t out_stride,
+    AttnForm form) {
   extern __shared__ float sm[];
-  const int kd = dim + 1;                             // padded key row: a lane per key reads its row without bank conflicts
-  float* s_k = sm;                                    // [64][dim + 1]
+  const int qd = MAPS * dim;                          // values of one query / key head (all maps)
+  const int kd = qd + 1;                              // padded key row: a lane per key reads its row without bank conflicts
+  float* s_k = sm;                                    // [64][qd + 1]
   float* s_v = s_k + kAttKeys * kd;                   // [64][vdim]
-  float* s_q = s_v + kAttKeys * vdim;                 // [16][dim]
-  float* s_p = s_q + kAttRows * dim;                  // [4 waves][64]
+  float* s_q = s_v + kAttKeys * vdim;                 // [16][qd]
+  float* s_p = s_q + kAttRows * qd;                   // [4 waves][MAPS][64]
   const int tile = blockIdx.x, g = blockIdx.y;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int row0 = tile_row0[tile], ntok = tile_ntok[tile], qh0 = tile_qh0[tile], nqh = tile_nqh[tile];
@@ -88,28 +116,34 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   const int e = row_entry[row0];
   const int32_t* pages = page_ids + page_indptr[e];
   const int kmax = positions[row0 + ntok - 1] + 1;    // keys 0 .. kmax - 1 are visible to the tile's last token
-  for (int i = tid; i < nrows * dim; i += 256) {
-    const int lr = i / dim, d = i % dim;
+  // the first key any row of the tile sees, rounded down to the 64-key grid that starts at position 0
+  const int kfirst = form.block > 0 ? ((positions[row0] / form.block) * form.block / kAttKeys) * kAttKeys : 0;
+  for (int i = tid; i < nrows * qd; i += 256) {
+    const int lr = i / qd, d = i % qd;
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
-    s_q[lr * dim + d] = q[((int64_t)(row0 + tok) * H + qh) * dim + d];
+    s_q[lr * qd + d] = q[((int64_t)(row0 + tok) * H + qh) * qd + d];
   }
-  float mrun[kAttRpw], lrun[kAttRpw], acc[kAttRpw][4];
-  int rpos[kAttRpw];
+  float mrun[kAttRpw][MAPS], lrun[kAttRpw][MAPS], acc[kAttRpw][MAPS][4];
+  int rpos[kAttRpw], rlo[kAttRpw];
 #pragma unroll
   for (int i = 0; i < kAttRpw; ++i) {
-    mrun[i] = -INFINITY;
-    lrun[i] = 0.f;
     const int lr = wave + 4 * i;
     rpos[i] = lr < nrows ? positions[row0 + lr / nqh] : -1;
+    rlo[i] = form.block > 0 && rpos[i] >= 0 ? (rpos[i] / form.block) * form.block : 0;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[i][c] = 0.f;
+    for (int m = 0; m < MAPS; ++m) {
+      mrun[i][m] = -INFINITY;
+      lrun[i][m] = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[i][m][c] = 0.f;
+    }
   }
-  for (int k0 = 0; k0 < kmax; k0 += kAttKeys) {
+  for (int k0 = kfirst; k0 < kmax; k0 += kAttKeys) {
     const int nk = min(kAttKeys, kmax - k0);
     __syncthreads();
-    for (int i = tid; i < nk * dim; i += 256) {
-      const int j = i / dim, d = i % dim, p = k0 + j;
-      s_k[j * kd + d] = ld(cache + (int64_t)pages[p / page_size] * page_stride + k_cache_off + ((int64_t)(p % page_size) * G + g) * dim + d);
+    for (int i = tid; i < nk * qd; i += 256) {
+      const int j = i / qd, d = i % qd, p = k0 + j;
+      s_k[j * kd + d] = ld(cache + (int64_t)pages[p / page_size] * page_stride + k_cache_off + ((int64_t)(p % page_size) * G + g) * qd + d);
     }
     for (int i = tid; i < nk * vdim; i += 256) {
       const int j = i / vdim, d = i % vdim, p = k0 + j;
@@ -119,34 +153,39 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
 #pragma unroll
     for (int i = 0; i < kAttRpw; ++i) {
       const int lr = wave + 4 * i;
-      if (lr >= nrows) continue;          // uniform over the wave
-      if (k0 > rpos[i]) continue;         // the whole tile lies after this row's position
-      float s = -INFINITY;
-      if (lane < nk && k0 + lane <= rpos[i]) {
-        float a = 0.f;
-        const float* kr = s_k + lane * kd;
-        const float* qr = s_q + lr * dim;
-        for (int d = 0; d < dim; ++d) a = fmaf(qr[d], kr[d], a);
-        s = a * scale;
-      }
-      const float mnew = fmaxf(mrun[i], wave_max(s));
-      const float p = s == -INFINITY ? 0.f : expf(s - mnew);
-      const float corr = mrun[i] == -INFINITY ? 0.f : expf(mrun[i] - mnew);
-      lrun[i] = lrun[i] * corr + wave_sum(p);
-      mrun[i] = mnew;
-      s_p[wave * 64 + lane] = p;
-      __builtin_amdgcn_wave_barrier();
-      const int jn = min(nk, rpos[i] - k0 + 1);
+      if (lr >= nrows) continue;                              // uniform over the wave
+      if (k0 > rpos[i] || k0 + nk <= rlo[i]) continue;        // the whole tile lies after this row's position or before its run
+      const bool seen = lane < nk && k0 + lane <= rpos[i] && k0 + lane >= rlo[i];
+      const int j0 = max(0, rlo[i] - k0), jn = min(nk, rpos[i] - k0 + 1);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const int col = lane + 64 * c;
-        if (col < vdim) {
-          float a = acc[i][c] * corr;
-          for (int j = 0; j < jn; ++j) a = fmaf(s_p[wave * 64 + j], s_v[j * vdim + col], a);
-          acc[i][c] = a;
+      for (int m = 0; m < MAPS; ++m) {
+        float s = -INFINITY;
+        if (seen) {
+          float a = 0.f;
+          const float* kr = s_k + lane * kd + m * dim;
+          const float* qr = s_q + lr * qd + m * dim;
+          for (int d = 0; d < dim; ++d) a = fmaf(qr[d], kr[d], a);
+          s = a * scale;
         }
+        const float mnew = fmaxf(mrun[i][m], wave_max(s));
+        const float p = s == -INFINITY ? 0.f : expf(s - mnew);
+        const float corr = mrun[i][m] == -INFINITY ? 0.f : expf(mrun[i][m] - mnew);
+        lrun[i][m] = lrun[i][m] * corr + wave_sum(p);
+        mrun[i][m] = mnew;
+        float* pw = s_p + (wave * MAPS + m) * 64;
+        pw[lane] = p;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const int col = lane + 64 * c;
+          if (col < vdim) {
+            float a = acc[i][m][c] * corr;
+            for (int j = j0; j < jn; ++j) a = fmaf(pw[j], s_v[j * vdim + col], a);
+            acc[i][m][c] = a;
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
       }
-      __builtin_amdgcn_wave_barrier();
     }
   }
 #pragma unroll
@@ -154,11 +193,39 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
     const int lr = wave + 4 * i;
     if (lr >= nrows) continue;
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
-    const float invl = factor / lrun[i];
+    float res[4];
+    if (form.sink) {   // the sink joins the denominator of every map: rescale to the larger of the two maxima first
+      const float sk = ld(static_cast<const A*>(form.sink) + qh);
+#pragma unroll
+      for (int m = 0; m < MAPS; ++m) {
+        const float mnew = fmaxf(mrun[i][m], sk);
+        const float corr = mrun[i][m] == -INFINITY ? 0.f : expf(mrun[i][m] - mnew);
+        lrun[i][m] = lrun[i][m] * corr + expf(sk - mnew);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[i][m][c] *= corr;
+      }
+    }
+    if constexpr (MAPS == 1) {
+      const float invl = 1.0f / lrun[i][0];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) res[c] = acc[i][0][c] * invl;
+    } else {
+      const float inv0 = 1.0f / lrun[i][0], inv1 = form.lambda / lrun[i][MAPS - 1];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) res[c] = acc[i][0][c] * inv0 - acc[i][MAPS - 1][c] * inv1;
+    }
+    float post = factor;
+    if (form.head_norm) {
+      float ss = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (lane + 64 * c < vdim) ss = fmaf(res[c], res[c], ss);
+      post = factor / sqrtf(wave_sum(ss) / (float)vdim + form.norm_eps);
+    }
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int col = lane + 64 * c;
-      if (col < vdim) st(out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim + col, acc[i][c] * invl);
+      if (col < vdim) st(out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim + col, res[c] * post);
     }
   }
 }
@@ -179,6 +246,31 @@ using namespace pk;
 
 #define PK_BAD ((pegainfer_status_t)hipErrorInvalidValue)
 
+pegainfer_status_t pegainfer_qk_prep_paged(const void* proj, int64_t proj_stride, int64_t q_off, int64_t k_off, int64_t v_off,
+                                          int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, const void* q_norm,
+                                          const void* k_norm, float eps, const void* q_bias, const void* k_bias,
+                                          const void* v_bias, float qt_coef, int32_t qt_every, const float* inv_freq,
+                                          int32_t rot_dims, const int32_t* positions, const int32_t* row_entry,
+                                          const int32_t* page_indptr, const int32_t* page_ids, void* cache, int64_t page_stride,
+                                          int64_t k_cache_off, int64_t v_cache_off, int32_t page_size, float* q_out,
+                                          void* q_out_stored, int32_t n_rows, int32_t dtype, pegainfer_stream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims > dim || (rot_dims & 1) || page_size <= 0 ||
+      (rot_dims > 0 && !inv_freq) || (!q_norm) != (!k_norm) || (size_t)4 * dim * sizeof(float) > 64 * 1024)
+    return PK_BAD;
+  if (!by_dtype(dtype, [&](auto* t) {
+        using A = std::remove_pointer_t<decltype(t)>;
+        qk_norm_rope_paged_kernel<A><<<n_rows, 256, (size_t)4 * dim * sizeof(float), as_stream(stream)>>>(
+            static_cast<const A*>(proj), proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim,
+            static_cast<const A*>(q_norm), static_cast<const A*>(k_norm), eps, inv_freq, rot_dims, positions, row_entry,
+            page_indptr, page_ids, static_cast<A*>(cache), page_stride, k_cache_off, v_cache_off, page_size, q_out,
+            static_cast<A*>(q_out_stored), static_cast<const A*>(q_bias), static_cast<const A*>(k_bias),
+            static_cast<const A*>(v_bias), qt_coef, qt_every);
+      }))
+    return PK_BAD;
+  return (pegainfer_status_t)hipGetLastError();
+}
+
 pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_stride, int64_t q_off, int64_t k_off,
                                                 int64_t v_off, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim,
                                                 const void* q_norm, const void* k_norm, float eps, const float* inv_freq,
@@ -187,19 +279,51 @@ pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_s
                                                 int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
                                                 int32_t page_size, float* q_out, void* q_out_stored, int32_t n_rows,
                                                 int32_t dtype, pegainfer_stream_t stream) {
-  if (n_rows <= 0) return 0;
-  if (heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims > dim || (rot_dims & 1) || page_size <= 0)
+  if (!q_norm || !k_norm) return PK_BAD;
+  return pegainfer_qk_prep_paged(proj, proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim, q_norm, k_norm, eps, nullptr,
+                                 nullptr, nullptr, 0.f, 0, inv_freq, rot_dims, positions, row_entry, page_indptr, page_ids, cache,
+                                 page_stride, k_cache_off, v_cache_off, page_size, q_out, q_out_stored, n_rows, dtype, stream);
+}
+
+pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
+                                                int64_t v_cache_off, int32_t page_size, const int32_t* positions,
+                                                const int32_t* row_entry, const int32_t* page_indptr, const int32_t* page_ids,
+                                                int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float scale,
+                                                float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
+                                                const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
+                                                int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
+                                                int32_t head_norm, float norm_eps, int32_t dtype, pegainfer_stream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || (maps != 1 && maps != 2) || maps * dim > 256 || vdim <= 0 ||
+      vdim > 256 || page_size <= 0 || kv_heads > 65535 || block < 0)
     return PK_BAD;
-  if (!by_dtype(dtype, [&](auto* t) {
-        using A = std::remove_pointer_t<decltype(t)>;
-        qk_norm_rope_paged_kernel<A><<<n_rows, 256, (size_t)4 * dim * sizeof(float), as_stream(stream)>>>(
-            static_cast<const A*>(proj), proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim,
-            static_cast<const A*>(q_norm), static_cast<const A*>(k_norm), eps, inv_freq, rot_dims, positions, row_entry,
-            page_indptr, page_ids, static_cast<A*>(cache), page_stride, k_cache_off, v_cache_off, page_size, q_out,
-            static_cast<A*>(q_out_stored));
-      }))
-    return PK_BAD;
-  return (pegainfer_status_t)hipGetLastError();
+  const int qd = maps * dim;
+  const size_t smem = ((size_t)kAttKeys * (qd + 1) + (size_t)kAttKeys * vdim + (size_t)kAttRows * qd + 4 * maps * 64) * sizeof(float);
+  const dim3 grid(n_tiles, kv_heads);
+  AttnForm form;
+  form.block = block;
+  form.sink = sink;
+  form.lambda = lambda;
+  form.head_norm = head_norm;
+  form.norm_eps = norm_eps;
+  bool ok = true;
+  const bool known = by_dtype(dtype, [&](auto* t) {
+    using A = std::remove_pointer_t<decltype(t)>;
+    auto go = [&](auto kern) {
+      if (smem > 48 * 1024 &&
+          hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+        ok = false;
+        return;
+      }
+      kern<<<grid, 256, smem, as_stream(stream)>>>(q, static_cast<const A*>(cache), page_stride, k_cache_off, v_cache_off,
+                                                   page_size, positions, row_entry, page_indptr, page_ids, heads, kv_heads, dim,
+                                                   vdim, scale, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh,
+                                                   static_cast<A*>(out), out_stride, form);
+    };
+    if (maps == 1) go(paged_attention_kernel<A, 1>);
+    else go(paged_attention_kernel<A, 2>);
+  });
+  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
 }
 
 pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
@@ -209,27 +333,9 @@ pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, 
                                              float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
                                              const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
                                              int64_t out_stride, int32_t dtype, pegainfer_stream_t stream) {
-  if (n_tiles <= 0) return 0;
-  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > 256 || vdim <= 0 || vdim > 256 || page_size <= 0 ||
-      kv_heads > 65535)
-    return PK_BAD;
-  const size_t smem = ((size_t)kAttKeys * (dim + 1) + (size_t)kAttKeys * vdim + (size_t)kAttRows * dim + 4 * 64) * sizeof(float);
-  const dim3 grid(n_tiles, kv_heads);
-  bool ok = true;
-  const bool known = by_dtype(dtype, [&](auto* t) {
-    using A = std::remove_pointer_t<decltype(t)>;
-    auto kern = paged_attention_kernel<A>;
-    if (smem > 48 * 1024 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
-      ok = false;
-      return;
-    }
-    kern<<<grid, 256, smem, as_stream(stream)>>>(q, static_cast<const A*>(cache), page_stride, k_cache_off, v_cache_off,
-                                                 page_size, positions, row_entry, page_indptr, page_ids, heads, kv_heads, dim,
-                                                 vdim, scale, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh,
-                                                 static_cast<A*>(out), out_stride);
-  });
-  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
+  return pegainfer_paged_attention_ex(q, cache, page_stride, k_cache_off, v_cache_off, page_size, positions, row_entry, page_indptr,
+                                      page_ids, heads, kv_heads, dim, vdim, scale, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh,
+                                      n_tiles, out, out_stride, 1, 0.f, 0, nullptr, 0, 0.f, dtype, stream);
 }
 
 pegainfer_status_t pegainfer_scale_rows(const void* in, int64_t in_stride, void* out, int64_t out_stride, int32_t cols,

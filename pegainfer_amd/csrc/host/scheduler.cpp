@@ -13,6 +13,7 @@
 #include "pegainfer_qwen35.h"
 #include "pegainfer_duguzen.h"
 #include "pegainfer_feruzen.h"
+#include "pegainfer_ramalix.h"
 #include "pegainfer_scheduler.h"
 
 namespace psched {
@@ -276,7 +277,7 @@ struct Qwen35Exec {
   }
 };
 
-// Executor over a runtime with ONE batched step function (pegainfer_duguzen.h, pegainfer_feruzen.h).  The step takes prompts
+// Executor over a runtime with ONE batched step function (pegainfer_duguzen.h, pegainfer_feruzen.h, pegainfer_ramalix.h).  The step takes prompts
 // and single tokens of several requests as ONE batch, so a Prefill, a Decode and a Unified plan are all the same call;
 // sampled requests draw from their wanted row afterwards, logprobs read the row's fp32 logits.  Api names the runtime's
 // entry points.
@@ -301,6 +302,7 @@ struct Qwen35Exec {
   }
 PEGAINFER_STEP_API(DuguzenApi, pegainfer_duguzen);
 PEGAINFER_STEP_API(FeruzenApi, pegainfer_feruzen);
+PEGAINFER_STEP_API(RamalixApi, pegainfer_ramalix);
 
 template <class Api>
 struct StepExec {
@@ -365,6 +367,7 @@ struct StepExec {
 };
 using DuguzenExec = StepExec<DuguzenApi>;
 using FeruzenExec = StepExec<FeruzenApi>;
+using RamalixExec = StepExec<RamalixApi>;
 
 struct Scheduler {
   pegainfer_executor_vtbl ex;
@@ -372,6 +375,7 @@ struct Scheduler {
   Qwen35Exec* owned35 = nullptr;
   DuguzenExec* owned_dz = nullptr;
   FeruzenExec* owned_fz = nullptr;
+  RamalixExec* owned_rx = nullptr;
   Rng rng;
   std::vector<Active> active;
   std::vector<Pending> deferred;
@@ -654,12 +658,26 @@ pegainfer_sched_t pegainfer_sched_create_feruzen(void* model, uint64_t seed, con
   s->owned_fz = e;
   return s;
 }
+pegainfer_sched_t pegainfer_sched_create_ramalix(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop) {
+  if (!model) return nullptr;
+  auto* e = new psched::RamalixExec();
+  e->model = model;
+  for (int i = 0; i < n_stop; ++i) e->stop.insert(stop_tokens[i]);
+  pegainfer_executor_vtbl v{sizeof(pegainfer_executor_vtbl), e, &psched::RamalixExec::page_size, &psched::RamalixExec::max_request_pages,
+                            &psched::RamalixExec::available_pages, &psched::RamalixExec::is_stop_token,
+                            &psched::RamalixExec::drop_request, &psched::RamalixExec::execute, &psched::RamalixExec::last_error,
+                            &psched::RamalixExec::max_batch_size, &psched::RamalixExec::logprobs, nullptr, nullptr};
+  Scheduler* s = static_cast<Scheduler*>(pegainfer_sched_create(&v, seed));
+  s->owned_rx = e;
+  return s;
+}
 void pegainfer_sched_destroy(pegainfer_sched_t s) {
   if (!s) return;
   delete SC(s)->owned;
   delete SC(s)->owned35;
   delete SC(s)->owned_dz;
   delete SC(s)->owned_fz;
+  delete SC(s)->owned_rx;
   delete SC(s);
 }
 uint64_t pegainfer_sched_submit_ex(pegainfer_sched_t s, const uint32_t* prompt_tokens, int32_t n_tokens, int32_t max_tokens,

@@ -8,7 +8,10 @@
 //   sort_kernel     (row, choice) pairs bucketed by expert with LDS counters, an exclusive scan, and the table of <= 64-row
 //                   tiles the grouped GEMM walks.  The order of pairs inside an expert comes from atomics; every pair owns
 //                   its output row, so results do not depend on it.  Tiles hold <= 64 or <= 128 rows, as the GEMM form that walks them wants.
-//   combine_kernel  out[row] = sum over the row's choices, in choice order, of weight * expert output (fp32 sum).
+//   combine_kernel  out[row] = sum over the row's choices, in choice order, of weight * expert output (fp32 sum), plus a row
+//                   every token gets (a shared expert), optionally times the sigmoid of a per-row gate logit.
+// Options of the selection: a group's score = its two largest choices (default) or its largest; the chosen weights as they
+// are (default) or divided by their sum.
 #include <algorithm>
 
 #include "common.h"
@@ -23,7 +26,7 @@ namespace pk {
 template <typename A>
 __device__ __forceinline__ void route_select_wave(float* s, float* ch, float* gs, const A* __restrict__ corr,
                                                   int32_t* __restrict__ out_e, float* __restrict__ out_w, int row, int lane, int E,
-                                                  int G, int keep, int top, int score) {
+                                                  int G, int keep, int top, int score, int group_kind = 0, int renorm = 0) {
   if (score == PEGAINFER_SCORE_SOFTMAX) {            // s = exp(z - max) / sum over ALL experts, then the choice scores
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
@@ -46,7 +49,7 @@ __device__ __forceinline__ void route_select_wave(float* s, float* ch, float* gs
         const float v = ch[g * per + i];
         if (v > b0) { b1 = b0; b0 = v; } else if (v > b1) b1 = v;
       }
-      gs[g] = per >= 2 ? b0 + b1 : b0;
+      gs[g] = per >= 2 && group_kind == PEGAINFER_GROUP_TOP2_SUM ? b0 + b1 : b0;
     }
     __builtin_amdgcn_wave_barrier();
     for (int g = lane; g < G; g += 64) {             // kept = fewer than `keep` groups rank ahead (ties: the lower index)
@@ -81,6 +84,12 @@ __device__ __forceinline__ void route_select_wave(float* s, float* ch, float* gs
       if (found) ch[be] = -INFINITY;
     }
     __builtin_amdgcn_wave_barrier();
+  }
+  if (renorm && lane == 0) {   // the chosen weights divided by their sum (in choice order)
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) sum += out_w[(size_t)row * top + k];
+    const float inv = 1.0f / (sum + 1e-20f);
+    for (int k = 0; k < top; ++k) out_w[(size_t)row * top + k] *= inv;
   }
 }
 
@@ -139,7 +148,8 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
 template <typename A>
 __global__ __launch_bounds__(256) void route_from_logits_kernel(const float* __restrict__ logits, const A* __restrict__ corr,
                                                                 int32_t* __restrict__ out_e, float* __restrict__ out_w, int E,
-                                                                int G, int keep, int top, int rows, int score) {
+                                                                int G, int keep, int top, int rows, int score,
+                                                                int64_t logits_stride, int group_kind, int renorm) {
   extern __shared__ float sm[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + wave;
@@ -148,13 +158,13 @@ __global__ __launch_bounds__(256) void route_from_logits_kernel(const float* __r
   float* ch = s + E;
   float* gs = s + 2 * E;
   for (int e = lane; e < E; e += 64) {
-    const float z = logits[(size_t)row * E + e];
+    const float z = logits[(size_t)row * logits_stride + e];
     const float sc = score == PEGAINFER_SCORE_SOFTMAX ? z : sigmoid_f(z);
     s[e] = sc;
     ch[e] = corr ? sc + ld(corr + e) : sc;
   }
   __builtin_amdgcn_wave_barrier();
-  route_select_wave(s, ch, gs, corr, out_e, out_w, row, lane, E, G, keep, top, score);
+  route_select_wave(s, ch, gs, corr, out_e, out_w, row, lane, E, G, keep, top, score, group_kind, renorm);
 }
 
 __global__ __launch_bounds__(256) void route_sort_kernel(const int32_t* __restrict__ expert, int n_pairs, int top, int E,
@@ -192,10 +202,12 @@ __global__ __launch_bounds__(256) void route_sort_kernel(const int32_t* __restri
 
 template <typename A>
 __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restrict__ y, const float* __restrict__ w,
-                                                            const A* __restrict__ add, A* __restrict__ out, int d, int top) {
+                                                            const A* __restrict__ add, A* __restrict__ out, int d, int top,
+                                                            const float* __restrict__ add_gate, int64_t add_gate_stride) {
   const int row = blockIdx.x;
+  const float gate = add && add_gate ? sigmoid_f(add_gate[(size_t)row * add_gate_stride]) : 1.0f;
   for (int i = blockIdx.y * 256 + threadIdx.x; i < d; i += gridDim.y * 256) {
-    float a = add ? ld(add + (size_t)row * d + i) : 0.f;
+    float a = add ? ld(add + (size_t)row * d + i) * gate : 0.f;
     for (int c = 0; c < top; ++c) a = fmaf(w[(size_t)row * top + c], y[((size_t)row * top + c) * d + i], a);
     st(out + (size_t)row * d + i, a);
   }
@@ -226,22 +238,33 @@ pegainfer_status_t pegainfer_route_topk(const void* h, const void* w_router, con
   return (pegainfer_status_t)hipGetLastError();
 }
 
-pegainfer_status_t pegainfer_route_from_logits(const float* logits, const void* correction, int32_t* out_expert, float* out_weight,
-                                               int32_t experts, int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
-                                               int32_t score_kind, int32_t dtype, pegainfer_stream_t stream) {
+pegainfer_status_t pegainfer_route_from_logits_ex(const float* logits, int64_t logits_stride, const void* correction,
+                                                  int32_t* out_expert, float* out_weight, int32_t experts, int32_t n_groups,
+                                                  int32_t keep_groups, int32_t top, int32_t rows, int32_t score_kind,
+                                                  int32_t group_kind, int32_t renorm, int32_t dtype, pegainfer_stream_t stream) {
   if (rows <= 0) return 0;
   if (n_groups < 1) n_groups = 1;
   if (experts <= 0 || experts % n_groups || top <= 0 || top > experts || keep_groups < 1 || keep_groups > n_groups ||
-      (size_t)(2 * experts + n_groups) * 16 > 60000 || (score_kind != PEGAINFER_SCORE_SIGMOID && score_kind != PEGAINFER_SCORE_SOFTMAX))
+      logits_stride < experts || (size_t)(2 * experts + n_groups) * 16 > 60000 ||
+      (score_kind != PEGAINFER_SCORE_SIGMOID && score_kind != PEGAINFER_SCORE_SOFTMAX) ||
+      (group_kind != PEGAINFER_GROUP_TOP2_SUM && group_kind != PEGAINFER_GROUP_MAX))
     return (pegainfer_status_t)hipErrorInvalidValue;
   const size_t smem = (size_t)4 * (2 * experts + n_groups) * sizeof(float);
   if (!by_dtype(dtype, [&](auto* t) {
         using A = std::remove_pointer_t<decltype(t)>;
         route_from_logits_kernel<A><<<ceil_div(rows, 4), 256, smem, as_stream(stream)>>>(
-            logits, static_cast<const A*>(correction), out_expert, out_weight, experts, n_groups, keep_groups, top, rows, score_kind);
+            logits, static_cast<const A*>(correction), out_expert, out_weight, experts, n_groups, keep_groups, top, rows, score_kind,
+            logits_stride, group_kind, renorm);
       }))
     return (pegainfer_status_t)hipErrorInvalidValue;
   return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_route_from_logits(const float* logits, const void* correction, int32_t* out_expert, float* out_weight,
+                                               int32_t experts, int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
+                                               int32_t score_kind, int32_t dtype, pegainfer_stream_t stream) {
+  return pegainfer_route_from_logits_ex(logits, experts, correction, out_expert, out_weight, experts, n_groups, keep_groups, top, rows,
+                                        score_kind, PEGAINFER_GROUP_TOP2_SUM, 0, dtype, stream);
 }
 
 pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_router, const void* correction,
@@ -265,18 +288,24 @@ pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, 
   return (pegainfer_status_t)hipGetLastError();
 }
 
-pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float* weight, const void* add, void* out, int32_t d,
-                                               int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream) {
+pegainfer_status_t pegainfer_route_combine_gated(const float* y_pairs, const float* weight, const void* add,
+                                                 const float* add_gate, int64_t add_gate_stride, void* out, int32_t d,
+                                                 int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream) {
   if (rows <= 0) return 0;
   if (!by_dtype(dtype, [&](auto* t) {
         using A = std::remove_pointer_t<decltype(t)>;
         // few rows (decoding): the row is cut over several workgroups
         const dim3 grid(rows, rows >= 256 ? 1 : std::min(16, ceil_div(d, 256)));
         route_combine_kernel<A><<<grid, 256, 0, as_stream(stream)>>>(y_pairs, weight, static_cast<const A*>(add),
-                                                                     static_cast<A*>(out), d, top);
+                                                                     static_cast<A*>(out), d, top, add_gate, add_gate_stride);
       }))
     return (pegainfer_status_t)hipErrorInvalidValue;
   return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float* weight, const void* add, void* out, int32_t d,
+                                               int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream) {
+  return pegainfer_route_combine_gated(y_pairs, weight, add, nullptr, 0, out, d, top, rows, dtype, stream);
 }
 
 pegainfer_status_t pegainfer_route_combine(const float* y_pairs, const float* weight, void* out, int32_t d, int32_t top,

@@ -81,7 +81,34 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(float* __restrict__ qkv
   }
 }
 
-template <int NS>
+// The same for a decay per (head, key channel): gates[row] = [g: heads * dim | beta: heads], the decay inputs come as an fp32
+// matrix `a` ([rows][heads * dim] at stride a_stride: the output of a low-rank projection pair), dt_bias has heads * dim values.
+template <typename A>
+__global__ __launch_bounds__(256) void delta_prep_channel_kernel(float* __restrict__ qkv, int64_t qkv_stride,
+                                                                 const A* __restrict__ proj, int64_t proj_stride, int64_t b_off,
+                                                                 const float* __restrict__ a, int64_t a_stride,
+                                                                 const A* __restrict__ A_log, const A* __restrict__ dt_bias,
+                                                                 float* __restrict__ gates, int H, int G, int dim) {
+  const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* qk = qkv + (int64_t)row * qkv_stride;
+  const float qs = 1.0f / sqrtf((float)dim);
+  for (int hh = wave; hh < 2 * G; hh += 4) {
+    float* x = qk + (int64_t)hh * dim;
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += 64) ss = fmaf(x[d], x[d], ss);
+    const float sc = (hh < G ? qs : 1.0f) / sqrtf(wave_sum(ss) + 1e-6f);
+    for (int d = lane; d < dim; d += 64) x[d] *= sc;
+  }
+  const A* pr = proj + (int64_t)row * proj_stride;
+  float* gr = gates + (int64_t)row * ((int64_t)H * dim + H);
+  for (int i = threadIdx.x; i < H * dim; i += 256)
+    gr[i] = expf(-expf(ld(A_log + i / dim)) * softplus_f(a[(int64_t)row * a_stride + i] + ld(dt_bias + i)));
+  for (int h = threadIdx.x; h < H; h += 256) gr[(int64_t)H * dim + h] = sigmoid_f(ld(pr + b_off + h));
+}
+
+// CH: the decay is one number per (head, key channel) - it scales the ROWS of S - and the gates row is laid out as
+// delta_prep_channel_kernel leaves it; otherwise one number per head ([g: heads | beta: heads]).
+template <int NS, bool CH>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int64_t qkv_stride,
                                                          const float* __restrict__ gates, float* __restrict__ state,
                                                          int64_t slot_stride, float* __restrict__ o, int H, int G, int dim,
@@ -90,6 +117,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
   constexpr int DP = kRecSlices * NS;
   __shared__ __attribute__((aligned(16))) float s_k[kRecTokens][DP], s_q[kRecTokens][DP];
   __shared__ float s_v[kRecTokens][kRecCols], s_g[kRecTokens], s_b[kRecTokens];
+  __shared__ __attribute__((aligned(16))) float s_gc[CH ? kRecTokens : 1][CH ? DP : 1];
+  const int64_t gs = CH ? (int64_t)H * dim + H : (int64_t)2 * H;   // floats of one gates row
   const int e = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kRecCols;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, cl = wave * 4 + (lane >> 4);
   const int col = col0 + cl;
@@ -116,8 +145,16 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     __syncthreads();
     nxt.land(tid, s_q, s_k, s_v);
     if (tid < kRecTokens) {   // rows past the entry's end: g = 1, beta = 0, zero key - a step that leaves S as it is
-      s_g[tid] = tid < tc ? gates[(int64_t)(row0 + t0 + tid) * 2 * H + h] : 1.f;
-      s_b[tid] = tid < tc ? gates[(int64_t)(row0 + t0 + tid) * 2 * H + H + h] : 0.f;
+      s_g[tid] = tid < tc && !CH ? gates[(int64_t)(row0 + t0 + tid) * gs + h] : 1.f;
+      s_b[tid] = tid < tc ? gates[(int64_t)(row0 + t0 + tid) * gs + (CH ? (int64_t)H * dim : H) + h] : 0.f;
+    }
+    if constexpr (CH) {
+      const int tt = tid >> 4, part = tid & 15;
+#pragma unroll
+      for (int j = 0; j < NS; ++j) {
+        const int d = part + 16 * j;
+        s_gc[tt][d] = tt < tc && d < dim ? gates[(int64_t)(row0 + t0 + tt) * gs + (int64_t)h * dim + d] : 1.f;
+      }
     }
     __syncthreads();
     if (t0 + kRecTokens < len) fetch(t0 + kRecTokens);
@@ -132,7 +169,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
 #pragma unroll
       for (int i = 0; i < NS; ++i) {
         kk[i] = s_k[tt][r * NS + i];
-        S[i] *= g;
+        if constexpr (CH) S[i] *= s_gc[tt][r * NS + i]; else S[i] *= g;
         if (i & 1) a1 = fmaf(S[i], kk[i], a1); else a0 = fmaf(S[i], kk[i], a0);
       }
       const float u = beta * (v - row16_sum(a0 + a1));
@@ -292,9 +329,35 @@ pegainfer_status_t pegainfer_delta_rule(float* qkv, int64_t qkv_stride, const vo
     return PK_BAD;
   const dim3 grid(ceil_div(vdim, kRecCols), heads, n_entries);
   if (!by_slices(dim, [&](auto ns) {
-        delta_rule_kernel<decltype(ns)::value><<<grid, 256, 0, as_stream(stream)>>>(qkv, qkv_stride, gates, state, slot_stride, o,
+        delta_rule_kernel<decltype(ns)::value, false><<<grid, 256, 0, as_stream(stream)>>>(qkv, qkv_stride, gates, state, slot_stride, o,
                                                                                     heads, kv_heads, dim, vdim, entry_row0,
                                                                                     entry_slot);
+      }))
+    return PK_BAD;
+  return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_delta_rule_channel(float* qkv, int64_t qkv_stride, const void* proj, int64_t proj_stride,
+                                                int64_t b_off, const float* a, int64_t a_stride, const void* A_log,
+                                                const void* dt_bias, float* gates, float* state, int64_t slot_stride, float* o,
+                                                int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t n_rows,
+                                                const int32_t* entry_row0, const int32_t* entry_slot, int32_t n_entries,
+                                                int32_t dtype, pegainfer_stream_t stream) {
+  if (n_entries <= 0 || n_rows <= 0) return 0;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > 256 || vdim <= 0 || heads > 65535 || n_entries > 65535)
+    return PK_BAD;
+  if (!by_dtype(dtype, [&](auto* t) {
+        using A = std::remove_pointer_t<decltype(t)>;
+        delta_prep_channel_kernel<A><<<n_rows, 256, 0, as_stream(stream)>>>(qkv, qkv_stride, static_cast<const A*>(proj), proj_stride,
+                                                                            b_off, a, a_stride, static_cast<const A*>(A_log),
+                                                                            static_cast<const A*>(dt_bias), gates, heads, kv_heads, dim);
+      }))
+    return PK_BAD;
+  const dim3 grid(ceil_div(vdim, kRecCols), heads, n_entries);
+  if (!by_slices(dim, [&](auto ns) {
+        delta_rule_kernel<decltype(ns)::value, true><<<grid, 256, 0, as_stream(stream)>>>(qkv, qkv_stride, gates, state, slot_stride, o,
+                                                                                          heads, kv_heads, dim, vdim, entry_row0,
+                                                                                          entry_slot);
       }))
     return PK_BAD;
   return (pegainfer_status_t)hipGetLastError();

@@ -7,6 +7,8 @@
 //                           sum over the streams of earlier layers (depth-weighted averaging) in one pass over the row
 //   clamp_glu_rows_kernel   g = min(gate, L), u = clamp(up, -L, L):  g sigmoid(alpha g) (u + 1)
 //   head_rms_gate_kernel    per-head RMS norm of a read-out * weight * silu / sigmoid gate * constant
+//   scalar_rms_add_kernel   residual sum with a constant factor (+ bias, + extra rows, + one extra vector), then an RMS norm
+//                           whose gain is a single number
 #include <algorithm>
 
 #include "common.h"
@@ -243,6 +245,62 @@ __global__ __launch_bounds__(256) void head_rms_gate_kernel(const float* __restr
   }
 }
 
+// Residual sum with a constant factor, then an RMS norm whose gain is ONE number:
+//   r = x_in + mult * (y + bias) + add_rows + add_vec            (every term but x_in optional)      -> x_out (fp32)
+//   n = r / sqrt(mean(r^2) + eps) * gain[0]                                                          -> n_out (fp32, optional)
+// x_in and x_out may name the same memory (an element is read, then written, by the same thread).  The row stays in
+// registers between the sum and the norm: one pass over memory.  NPT: values a thread keeps (d <= 256 * NPT), 0 = any d
+// (the row is summed a second time instead).
+template <typename Y, typename A, int NPT>
+__global__ __launch_bounds__(256) void scalar_rms_add_kernel(const float* x_in, const Y* __restrict__ y, const A* __restrict__ bias,
+                                                             float mult, const float* __restrict__ add_rows,
+                                                             const A* __restrict__ add_vec, float* x_out,
+                                                             const A* __restrict__ gain, float eps, float* __restrict__ n_out,
+                                                             int d) {
+  __shared__ float red[4];
+  const int row = blockIdx.x;
+  const int64_t base = (int64_t)row * d;
+  auto value = [&](int i) {
+    float r = x_in[base + i];
+    if (y) r = fmaf(mult, ld(y + base + i) + (bias ? ld(bias + i) : 0.f), r);
+    if (add_rows) r += add_rows[base + i];
+    if (add_vec) r += ld(add_vec + i);
+    return r;
+  };
+  float ss = 0.f;
+  if constexpr (NPT > 0) {
+    float keep[NPT];
+#pragma unroll
+    for (int k = 0; k < NPT; ++k) {
+      const int i = threadIdx.x + 256 * k;
+      keep[k] = i < d ? value(i) : 0.f;
+      ss = fmaf(keep[k], keep[k], ss);
+    }
+    ss = block_sum<4>(ss, red);
+    const float sc = gain ? ld(gain) / sqrtf(ss / (float)d + eps) : 0.f;
+#pragma unroll
+    for (int k = 0; k < NPT; ++k) {
+      const int i = threadIdx.x + 256 * k;
+      if (i < d) {
+        if (x_out) x_out[base + i] = keep[k];
+        if (n_out) n_out[base + i] = keep[k] * sc;
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < d; i += 256) {
+      const float r = value(i);
+      ss = fmaf(r, r, ss);
+    }
+    ss = block_sum<4>(ss, red);   // its barriers also order every read of x_in before the writes below
+    const float sc = gain ? ld(gain) / sqrtf(ss / (float)d + eps) : 0.f;
+    for (int i = threadIdx.x; i < d; i += 256) {
+      const float r = value(i);
+      if (x_out) x_out[base + i] = r;
+      if (n_out) n_out[base + i] = r * sc;
+    }
+  }
+}
+
 }  // namespace pk
 
 extern "C" {
@@ -378,6 +436,31 @@ pegainfer_status_t pegainfer_head_rms_gate(const float* o, const void* w, int32_
       }))
     return PK_BAD;
   return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_scalar_rms_add(const float* x_in, const void* y, int32_t y_dtype, const void* bias, float mult,
+                                            const float* add_rows, const void* add_vec, float* x_out, const void* gain,
+                                            float eps, float* n_out, int32_t d, int32_t rows, int32_t dtype,
+                                            pegainfer_stream_t stream) {
+  if (rows <= 0) return 0;
+  if (d <= 0 || !x_in || (!x_out && !n_out) || (n_out && !gain)) return PK_BAD;
+  bool ok = true;
+  const bool known = by_dtype(y ? y_dtype : dtype, [&](auto* ty) {
+    using Y = std::remove_pointer_t<decltype(ty)>;
+    ok = by_dtype(dtype, [&](auto* ta) {
+      using A = std::remove_pointer_t<decltype(ta)>;
+      auto go = [&](auto npt) {
+        scalar_rms_add_kernel<Y, A, decltype(npt)::value><<<rows, 256, 0, as_stream(stream)>>>(
+            x_in, static_cast<const Y*>(y), static_cast<const A*>(bias), mult, add_rows, static_cast<const A*>(add_vec), x_out,
+            static_cast<const A*>(gain), eps, n_out, d);
+      };
+      if (d <= 1024) go(std::integral_constant<int, 4>());
+      else if (d <= 4096) go(std::integral_constant<int, 16>());
+      else if (d <= 8192) go(std::integral_constant<int, 32>());
+      else go(std::integral_constant<int, 0>());
+    });
+  });
+  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
 }
 
 }  // extern "C"

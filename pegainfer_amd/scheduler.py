@@ -59,7 +59,8 @@ class Scheduler:
         st = np.ascontiguousarray(list(stop_tokens), dtype=np.uint32)
         create = {"Qwen35Engine": lib.pegainfer_sched_create_qwen35,
                   "DuguzenEngine": lib.pegainfer_sched_create_duguzen,
-                  "FeruzenEngine": lib.pegainfer_sched_create_feruzen}.get(type(engine).__name__, lib.pegainfer_sched_create_qwen3)
+                  "FeruzenEngine": lib.pegainfer_sched_create_feruzen,
+                  "RamalixEngine": lib.pegainfer_sched_create_ramalix}.get(type(engine).__name__, lib.pegainfer_sched_create_qwen3)
         h = create(engine.h, seed, st.ctypes.data if st.size else None, int(st.size))
         return cls(h, keep=engine)
 
