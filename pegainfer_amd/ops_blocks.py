@@ -82,13 +82,13 @@ def gemm_strided(desc):
 
 
 def linear(x, w, out_dtype=None, epilogue=EPI_NONE, plain=False):
-    """y[T, M] = x[T, K] w[M, K]^T through pegainfer_gemm_strided (any sizes, bf16 or fp32 operands, fp32 accumulation);
-    plain = the fp32-FMA tile kernel whatever the shape"""
+    """y[T, M] = x[T, K] w[M, K]^T through pegainfer_gemm_strided (any sizes, bf16 or fp32 operands, fp32 accumulation; x may be
+    a column range of a wider matrix); plain = the fp32-FMA tile kernel whatever the shape"""
     T, K = x.shape
     M = w.shape[0]
     y = torch.empty((T, M), dtype=out_dtype or x.dtype, device=x.device)
     d = GemmDesc(x=_p(x), w=_p(w), y=_p(y), x_dtype=_dt(x), w_dtype=_dt(w), y_dtype=_dt(y), m=M, k=K, rows=T, groups=1,
-                 x_row_stride=K, w_m_stride=K, w_k_stride=1, y_row_stride=M, epilogue=epilogue, plain=int(plain))
+                 x_row_stride=x.stride(0), w_m_stride=K, w_k_stride=1, y_row_stride=M, epilogue=epilogue, plain=int(plain))
     gemm_strided(d)
     return y
 
@@ -316,4 +316,81 @@ def paged_attention(q, cache, page_stride, k_off, v_off, page_size, rg, page_ind
                                              _p(rg.row_entry), _p(page_indptr), _p(page_ids), H, kv_heads, dim, vdim,
                                              float(scale), float(factor), _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), t[0].numel(),
                                              _p(out), out.stride(0), _dt(cache), _stream()), "paged_attention")
+    return out
+
+
+# ---- one-number RMS gains, attention with options, channel decays, group-limited routing ----
+def scalar_rms_add(x, gain, eps, y=None, bias=None, mult=1.0, add_rows=None, add_vec=None, norm=True):
+    """r = x + mult (y + bias) + add_rows + add_vec (fp32), n = r / rms(r) * gain[0] (fp32) -> (r, n or None);
+    x fp32 [rows, d]; y / bias / add_vec / gain in the storage type of gain"""
+    rows, d = x.shape
+    r = torch.empty_like(x)
+    n = torch.empty_like(x) if norm else None
+    _chk(ffi.lib().pegainfer_scalar_rms_add(_p(x), _p(y), _dt(y) if y is not None else _dt(gain), _p(bias), float(mult), _p(add_rows),
+                                            _p(add_vec), _p(r), _p(gain) if norm else None, float(eps), _p(n), d, rows, _dt(gain),
+                                            _stream()), "scalar_rms_add")
+    return r, n
+
+
+def qk_prep_paged(proj, offs, heads, kv_heads, dim, vdim, rg, page_indptr, page_ids, cache, page_stride, k_off, v_off, page_size,
+                  q_norm=None, k_norm=None, eps=0.0, q_bias=None, k_bias=None, v_bias=None, qt_coef=0.0, qt_every=0, inv_freq=None,
+                  rot_dims=0):
+    """queries -> fp32 [rows, heads, dim]; keys and values -> the cache entry of (request, position).  dim counts ALL values of
+    a query / key head (both maps of a two-map attention)"""
+    q = torch.empty((proj.shape[0], heads, dim), dtype=torch.float32, device=proj.device)
+    _chk(ffi.lib().pegainfer_qk_prep_paged(_p(proj), proj.stride(0), offs[0], offs[1], offs[2], heads, kv_heads, dim, vdim, _p(q_norm),
+                                           _p(k_norm), float(eps), _p(q_bias), _p(k_bias), _p(v_bias), float(qt_coef), int(qt_every),
+                                           _p(inv_freq), rot_dims, _p(rg.positions), _p(rg.row_entry), _p(page_indptr), _p(page_ids),
+                                           _p(cache), page_stride, k_off, v_off, page_size, _p(q), None, proj.shape[0], _dt(proj),
+                                           _stream()), "qk_prep_paged")
+    return q
+
+
+def paged_attention_ex(q, cache, page_stride, k_off, v_off, page_size, rg, page_indptr, page_ids, kv_heads, vdim, scale, factor=1.0,
+                       maps=1, lam=0.0, block=0, sink=None, head_norm=False, norm_eps=0.0):
+    """q fp32 [rows, heads, maps * dim]"""
+    T, H, qd = q.shape
+    out = torch.empty((T, H * vdim), dtype=cache.dtype, device=q.device)
+    t = attention_tiles(rg.lens, H // kv_heads, q.device)
+    _chk(ffi.lib().pegainfer_paged_attention_ex(_p(q), _p(cache), page_stride, k_off, v_off, page_size, _p(rg.positions),
+                                                _p(rg.row_entry), _p(page_indptr), _p(page_ids), H, kv_heads, qd // maps, vdim,
+                                                float(scale), float(factor), _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), t[0].numel(),
+                                                _p(out), out.stride(0), maps, float(lam), int(block), _p(sink), int(bool(head_norm)),
+                                                float(norm_eps), _dt(cache), _stream()), "paged_attention_ex")
+    return out
+
+
+def delta_rule_channel(qkv_f32, proj, b_off, a_f32, A_log, dt_bias, state, heads, kv_heads, dim, vdim, rg):
+    """the gated delta rule with a decay per (head, key channel); a_f32 [rows, heads * dim] the decay inputs; otherwise as
+    delta_rule"""
+    o = torch.empty((qkv_f32.shape[0], heads * vdim), dtype=torch.float32, device=proj.device)
+    gates = torch.empty((qkv_f32.shape[0], heads * dim + heads), dtype=torch.float32, device=proj.device)
+    _chk(ffi.lib().pegainfer_delta_rule_channel(_p(qkv_f32), qkv_f32.stride(0), _p(proj), proj.stride(0), b_off, _p(a_f32),
+                                                a_f32.stride(0), _p(A_log), _p(dt_bias), _p(gates), _p(state), state.stride(0), _p(o),
+                                                heads, kv_heads, dim, vdim, qkv_f32.shape[0], _p(rg.entry_row0), _p(rg.entry_slot),
+                                                rg.n, _dt(proj), _stream()), "delta_rule_channel")
+    return o
+
+
+def route_from_logits_ex(logits_f32, experts, top, n_groups=1, keep_groups=1, score="softmax", group="max", renorm=True,
+                         dtype=torch.bfloat16):
+    """logits fp32 [rows, >= experts] (columns beyond `experts` are not read)"""
+    rows = logits_f32.shape[0]
+    e = torch.empty((rows, top), dtype=torch.int32, device=logits_f32.device)
+    w = torch.empty((rows, top), dtype=torch.float32, device=logits_f32.device)
+    _chk(ffi.lib().pegainfer_route_from_logits_ex(_p(logits_f32), logits_f32.stride(0), None, _p(e), _p(w), experts, n_groups,
+                                                  keep_groups, top, rows, 1 if score == "softmax" else 0, 1 if group == "max" else 0,
+                                                  int(bool(renorm)), 0 if dtype == torch.bfloat16 else 1, _stream()),
+         "route_from_logits_ex")
+    return e, w
+
+
+def route_combine_gated(y_pairs, weight, add, add_gate_f32, out_dtype):
+    """sum_c weight[row, c] y_pairs[row * top + c] + sigmoid(add_gate[row]) * add[row]; add_gate: an fp32 [rows] view (stride free)"""
+    rows, top = weight.shape
+    d = y_pairs.shape[1]
+    out = torch.empty((rows, d), dtype=out_dtype, device=y_pairs.device)
+    _chk(ffi.lib().pegainfer_route_combine_gated(_p(y_pairs), _p(weight), _p(add), _p(add_gate_f32),
+                                                 0 if add_gate_f32 is None else add_gate_f32.stride(0), _p(out), d, top, rows,
+                                                 _dt(out), _stream()), "route_combine_gated")
     return out
