@@ -94,6 +94,45 @@ struct AttnForm {
   float norm_eps = 0.f;
 };
 
+// A row's softmax states (one per map) turned into its output: the sink joins every denominator, the maps are combined, the
+// head is normed, `factor` comes last.  The wave holds the row: lane l has columns l, l + 64, ...
+template <typename A, int MAPS>
+__device__ __forceinline__ void attn_finish_row(float* mrun, float* lrun, float (*acc)[4], const AttnForm& form, int qh, int vdim,
+                                                float factor, int lane, A* __restrict__ dst) {
+  float res[4];
+  if (form.sink) {   // rescale to the larger of the two maxima first
+    const float sk = ld(static_cast<const A*>(form.sink) + qh);
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      const float mnew = fmaxf(mrun[m], sk);
+      const float corr = mrun[m] == -INFINITY ? 0.f : expf(mrun[m] - mnew);
+      lrun[m] = lrun[m] * corr + expf(sk - mnew);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[m][c] *= corr;
+    }
+  }
+  if constexpr (MAPS == 1) {
+    const float invl = 1.0f / lrun[0];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) res[c] = acc[0][c] * invl;
+  } else {
+    const float inv0 = 1.0f / lrun[0], inv1 = form.lambda / lrun[MAPS - 1];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) res[c] = acc[0][c] * inv0 - acc[MAPS - 1][c] * inv1;
+  }
+  float post = factor;
+  if (form.head_norm) {
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (lane + 64 * c < vdim) ss = fmaf(res[c], res[c], ss);
+    post = factor / sqrtf(wave_sum(ss) / (float)vdim + form.norm_eps);
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    if (lane + 64 * c < vdim) st(dst + lane + 64 * c, res[c] * post);
+}
+
 template <typename A, int MAPS>
 __global__ __launch_bounds__(256) void paged_attention_kernel(
     const float* __restrict__ q, const A* __restrict__ cache, int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
@@ -101,7 +140,7 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
     const int32_t* __restrict__ page_indptr, const int32_t* __restrict__ page_ids, int H, int G, int dim, int vdim, float scale,
     float factor, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ tile_ntok,
     const int32_t* __restrict__ tile_qh0, const int32_t* __restrict__ tile_nqh, A* __restrict__ out, int64_t out_stride,
-    AttnForm form) {
+    AttnForm form, int nsplit, float* __restrict__ part) {
   extern __shared__ float sm[];
   const int qd = MAPS * dim;                          // values of one query / key head (all maps)
   const int kd = qd + 1;                              // padded key row: a lane per key reads its row without bank conflicts
@@ -138,7 +177,9 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
       for (int c = 0; c < 4; ++c) acc[i][m][c] = 0.f;
     }
   }
-  for (int k0 = kfirst; k0 < kmax; k0 += kAttKeys) {
+  // nsplit > 1: workgroup z of the tile takes key tiles z, z + nsplit, ... (the count of splits does not depend on the
+  // context's length, so a recorded launch serves every later length) and leaves its softmax state to the merge kernel
+  for (int k0 = kfirst + (int)blockIdx.z * kAttKeys; k0 < kmax; k0 += kAttKeys * nsplit) {
     const int nk = min(kAttKeys, kmax - k0);
     __syncthreads();
     for (int i = tid; i < nk * qd; i += 256) {
@@ -188,45 +229,68 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
       }
     }
   }
+  if (nsplit > 1) {   // [tile][kv head][split][row][map][vdim values | maximum | sum]
+    float* pb = part + (((int64_t)(tile * G + g) * nsplit + blockIdx.z) * kAttRows) * MAPS * (vdim + 2);
+#pragma unroll
+    for (int i = 0; i < kAttRpw; ++i) {
+      const int lr = wave + 4 * i;
+      if (lr >= nrows) continue;
+#pragma unroll
+      for (int m = 0; m < MAPS; ++m) {
+        float* pr = pb + ((int64_t)lr * MAPS + m) * (vdim + 2);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (lane + 64 * c < vdim) pr[lane + 64 * c] = acc[i][m][c];
+        if (lane == 0) { pr[vdim] = mrun[i][m]; pr[vdim + 1] = lrun[i][m]; }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < kAttRpw; ++i) {
     const int lr = wave + 4 * i;
     if (lr >= nrows) continue;
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
-    float res[4];
-    if (form.sink) {   // the sink joins the denominator of every map: rescale to the larger of the two maxima first
-      const float sk = ld(static_cast<const A*>(form.sink) + qh);
+    attn_finish_row<A, MAPS>(mrun[i], lrun[i], acc[i], form, qh, vdim, factor, lane,
+                             out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
+  }
+}
+
+// The states that the splits of a tile have left, folded in split order, then finished like an unsplit row.
+template <typename A, int MAPS>
+__global__ __launch_bounds__(256) void paged_attention_merge_kernel(
+    const float* __restrict__ part, int nsplit, int H, int G, int vdim, float factor, const int32_t* __restrict__ tile_row0,
+    const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ tile_qh0, const int32_t* __restrict__ tile_nqh,
+    A* __restrict__ out, int64_t out_stride, AttnForm form) {
+  const int tile = blockIdx.x, g = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row0 = tile_row0[tile], ntok = tile_ntok[tile], qh0 = tile_qh0[tile], nqh = tile_nqh[tile];
+  const int nrows = ntok * nqh, per_group = H / G;
+  for (int lr = wave; lr < nrows; lr += 4) {
+    float mrun[MAPS], lrun[MAPS], acc[MAPS][4];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      mrun[m] = -INFINITY;
+      lrun[m] = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[m][c] = 0.f;
+    }
+    for (int z = 0; z < nsplit; ++z) {
 #pragma unroll
       for (int m = 0; m < MAPS; ++m) {
-        const float mnew = fmaxf(mrun[i][m], sk);
-        const float corr = mrun[i][m] == -INFINITY ? 0.f : expf(mrun[i][m] - mnew);
-        lrun[i][m] = lrun[i][m] * corr + expf(sk - mnew);
+        const float* pr = part + ((((int64_t)(tile * G + g) * nsplit + z) * kAttRows + lr) * MAPS + m) * (vdim + 2);
+        const float mz = pr[vdim], lz = pr[vdim + 1];
+        if (mz == -INFINITY) continue;     // a split that met no visible key
+        const float mnew = fmaxf(mrun[m], mz);
+        const float c0 = mrun[m] == -INFINITY ? 0.f : expf(mrun[m] - mnew), c1 = expf(mz - mnew);
+        lrun[m] = lrun[m] * c0 + lz * c1;
+        mrun[m] = mnew;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[i][m][c] *= corr;
+        for (int c = 0; c < 4; ++c)
+          if (lane + 64 * c < vdim) acc[m][c] = acc[m][c] * c0 + pr[lane + 64 * c] * c1;
       }
     }
-    if constexpr (MAPS == 1) {
-      const float invl = 1.0f / lrun[i][0];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) res[c] = acc[i][0][c] * invl;
-    } else {
-      const float inv0 = 1.0f / lrun[i][0], inv1 = form.lambda / lrun[i][MAPS - 1];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) res[c] = acc[i][0][c] * inv0 - acc[i][MAPS - 1][c] * inv1;
-    }
-    float post = factor;
-    if (form.head_norm) {
-      float ss = 0.f;
-#pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (lane + 64 * c < vdim) ss = fmaf(res[c], res[c], ss);
-      post = factor / sqrtf(wave_sum(ss) / (float)vdim + form.norm_eps);
-    }
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int col = lane + 64 * c;
-      if (col < vdim) st(out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim + col, res[c] * post);
-    }
+    const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
+    attn_finish_row<A, MAPS>(mrun, lrun, acc, form, qh, vdim, factor, lane, out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
   }
 }
 
@@ -292,14 +356,17 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
                                                 float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
                                                 const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
                                                 int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
-                                                int32_t head_norm, float norm_eps, int32_t dtype, pegainfer_stream_t stream) {
+                                                int32_t head_norm, float norm_eps, int32_t n_split, float* workspace,
+                                                int32_t dtype, pegainfer_stream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (n_split < 1) n_split = 1;
+  if (n_split > 1 && (!workspace || n_split > 65535)) return PK_BAD;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || (maps != 1 && maps != 2) || maps * dim > 256 || vdim <= 0 ||
       vdim > 256 || page_size <= 0 || kv_heads > 65535 || block < 0)
     return PK_BAD;
   const int qd = maps * dim;
   const size_t smem = ((size_t)kAttKeys * (qd + 1) + (size_t)kAttKeys * vdim + (size_t)kAttRows * qd + 4 * maps * 64) * sizeof(float);
-  const dim3 grid(n_tiles, kv_heads);
+  const dim3 grid(n_tiles, kv_heads, n_split);
   AttnForm form;
   form.block = block;
   form.sink = sink;
@@ -318,12 +385,25 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
       kern<<<grid, 256, smem, as_stream(stream)>>>(q, static_cast<const A*>(cache), page_stride, k_cache_off, v_cache_off,
                                                    page_size, positions, row_entry, page_indptr, page_ids, heads, kv_heads, dim,
                                                    vdim, scale, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh,
-                                                   static_cast<A*>(out), out_stride, form);
+                                                   static_cast<A*>(out), out_stride, form, n_split, workspace);
     };
-    if (maps == 1) go(paged_attention_kernel<A, 1>);
-    else go(paged_attention_kernel<A, 2>);
+    auto merge = [&](auto kern) {
+      kern<<<dim3(n_tiles, kv_heads), 256, 0, as_stream(stream)>>>(workspace, n_split, heads, kv_heads, vdim, factor, tile_row0,
+                                                                    tile_ntok, tile_qh0, tile_nqh, static_cast<A*>(out), out_stride, form);
+    };
+    if (maps == 1) {
+      go(paged_attention_kernel<A, 1>);
+      if (ok && n_split > 1) merge(paged_attention_merge_kernel<A, 1>);
+    } else {
+      go(paged_attention_kernel<A, 2>);
+      if (ok && n_split > 1) merge(paged_attention_merge_kernel<A, 2>);
+    }
   });
   return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
+}
+
+int64_t pegainfer_paged_attention_workspace(int32_t n_tiles, int32_t kv_heads, int32_t vdim, int32_t maps, int32_t n_split) {
+  return n_split > 1 ? (int64_t)n_tiles * kv_heads * n_split * kAttRows * maps * (vdim + 2) : 0;
 }
 
 pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
@@ -335,7 +415,7 @@ pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, 
                                              int64_t out_stride, int32_t dtype, pegainfer_stream_t stream) {
   return pegainfer_paged_attention_ex(q, cache, page_stride, k_cache_off, v_cache_off, page_size, positions, row_entry, page_indptr,
                                       page_ids, heads, kv_heads, dim, vdim, scale, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh,
-                                      n_tiles, out, out_stride, 1, 0.f, 0, nullptr, 0, 0.f, dtype, stream);
+                                      n_tiles, out, out_stride, 1, 0.f, 0, nullptr, 0, 0.f, 1, nullptr, dtype, stream);
 }
 
 pegainfer_status_t pegainfer_scale_rows(const void* in, int64_t in_stride, void* out, int64_t out_stride, int32_t cols,

@@ -82,6 +82,8 @@ static inline float host_bf2f(uint16_t h) {
 
 constexpr int kPageSize = 16;   // tokens per cache page, as in the other runtimes
 constexpr int kAttRows = 16;    // (token, query head) rows of one attention workgroup
+constexpr int kSplitGroups = 512;   // most (tile, kv head, key split) workgroups of an attention launch that cuts its keys
+constexpr int kMaxSplits = 16;
 
 enum { kDiffAttn = 1, kBlockAttn = 2, kChannelDelta = 3 };
 struct AttnCfg {
@@ -168,6 +170,8 @@ struct Model {
   float* tap = nullptr;
   size_t tap_cap = 0;
   int tap_rows = 0;
+  float* att_part = nullptr;   // softmax states of the key splits of an attention launch
+  int mx_vdim = 0;
   int mx_proj = 0, mx_mix = 0, mx_conv = 0, mx_q = 0, mx_o = 0, mx_gates = 0, mx_a = 0, mx_ff = 0, mx_top = 0, mx_gu_e = 0, mx_experts = 0;
 
   struct GraphKey {
@@ -362,6 +366,7 @@ struct Model {
         mx_a = std::max(mx_a, c.dl.heads * c.dl.dim);
       } else {
         mx_q = std::max(mx_q, c.at.heads * c.at.maps * c.at.dim);
+        mx_vdim = std::max(mx_vdim, c.at.vdim);
       }
       if (c.mlp.kind == 2) {
         mx_top = std::max(mx_top, c.mlp.top);
@@ -721,7 +726,8 @@ struct Model {
         dalloc(&a32, n * (size_t)std::max(1, mx_a), so) || dalloc(&o32, n * (size_t)std::max(1, mx_o), so) || dalloc_a(&hb, n * D, so) ||
         dalloc_a(&proj, n * (size_t)mx_proj, so) || dalloc_a(&mix, n * (size_t)mx_mix, so) || dalloc_a(&y, n * D, so) ||
         dalloc_a(&gate_d, n * (size_t)std::max(1, mx_o), so) || dalloc_a(&gu, n * (size_t)std::max(1, 2 * mx_ff), so) ||
-        dalloc_a(&act, n * (size_t)std::max(1, mx_ff), so) || dalloc_a(&ys, n * D, so))
+        dalloc_a(&act, n * (size_t)std::max(1, mx_ff), so) || dalloc_a(&ys, n * D, so) ||
+        dalloc(&att_part, (size_t)kSplitGroups * kAttRows * 2 * (size_t)(mx_vdim + 2), so))
       return -1;
     if (mx_top > 0 && (dalloc(&ypairs, P * D, so) || dalloc(&route_w, P, so) || dalloc(&route_logits, n * (size_t)(mx_experts + 1), so) ||
                        dalloc(&route_e, P, so) || dalloc(&pos_pair, P, so) || dalloc(&pos_row, P, so) ||
@@ -970,10 +976,14 @@ struct Model {
                                      w.v_bias, a.qt_coef, a.qt_every, w.inv_freq, a.rot_dims, d_pos, d_ent, d_ind, d_pages, cache,
                                      page_stride, r.k_off, r.v_off, kPageSize, q32, nullptr, Ti, dtype, S()));
         const bool two = a.maps == 2;
+        // a step of few rows (decoding, short portions) cannot fill the chip with one workgroup per (row tile, kv head): its
+        // keys are dealt to several workgroups.  The count depends on the step's shape only, never on the contexts' lengths.
+        const int wgs = (int)tile_cnt[ts] * a.kv;
+        const int nsplit = wgs >= 128 ? 1 : std::max(1, std::min(kMaxSplits, kSplitGroups / wgs));
         RX_K(pegainfer_paged_attention_ex(q32, cache, page_stride, r.k_off, r.v_off, kPageSize, d_pos, d_ent, d_ind, d_pages, a.heads,
                                           a.kv, a.dim, a.vdim, a.scale, two ? 1.0f - a.diff : 1.0f, tb, tb + tile_cnt[ts],
                                           tb + 2 * tile_cnt[ts], tb + 3 * tile_cnt[ts], (int)tile_cnt[ts], mix, c.mix_cols, a.maps,
-                                          w.lambda, a.block, w.sink, two ? 1 : 0, eps, dtype, S()));
+                                          w.lambda, a.block, w.sink, two ? 1 : 0, eps, nsplit, att_part, dtype, S()));
       }
       if (linear(w.o, mix, y, D, Ti, c.mix_cols)) return -1;
       // what the launch that closes this run norms for: the next run's first sublayer, unless that run opens a pass (its own

@@ -161,6 +161,37 @@ def marked_keys(n, d, dv, marks, askers, seed=2):
     return proj
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_split", [2, 5, 16])
+def test_key_splits_agree_with_the_unsplit_launch(dtype, n_split):
+    """decoding over a long context deals a row's key tiles to several workgroups and folds their softmax states: both attention
+    forms, splits that get no tile at all (16 splits over 3 key tiles), a block that begins in the middle of a key tile"""
+    Bk = B()
+    cfg = C.config_wide_heads()
+    w = C.random_weights(cfg, 7)
+    n = 150
+    h = C.bf16_round(torch.randn(n, cfg["width"], generator=torch.Generator().manual_seed(11)))
+    for li, maps in ((2, 2), (0, 1)):
+        p, m = "l%d.mix" % li, cfg["layers"][li]["mixer"]
+        H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        qd = maps * d
+        pc = Paged(PAGES, G, qd, dv, dtype)
+        proj = Bk.linear(dev(h, dtype), dev(torch.cat([w[p + ".q"], w[p + ".k"], w[p + ".v"]]), dtype), plain=True)
+        offs = [0, H * qd, (H + G) * qd]
+        rg = Bk.Ragged([n])
+        Bk.qk_prep_paged(proj, offs, H, G, qd, dv, rg, pc.indptr, pc.pids, pc.cache, pc.page_stride, pc.k_off, pc.v_off, 16)
+        form = dict(maps=2, lam=0.37, head_norm=True, norm_eps=1e-5, factor=0.3) if maps == 2 else \
+            dict(block=50, sink=dev(w[p + ".sink"], dtype))
+        for at in (n - 1, 127, 128, 3):          # single rows at several positions, as decoding brings them
+            one = Bk.Ragged([1], starts=[at])
+            q = Bk.qk_prep_paged(proj[at:at + 1], offs, H, G, qd, dv, one, pc.indptr, pc.pids, pc.cache, pc.page_stride, pc.k_off,
+                                 pc.v_off, 16)
+            args = (q, pc.cache, pc.page_stride, pc.k_off, pc.v_off, 16, one, pc.indptr, pc.pids, G, dv, m["scale"])
+            whole = Bk.paged_attention_ex(*args, **form)
+            cut = Bk.paged_attention_ex(*args, n_split=n_split, **form)
+            close(cut, whole.double().cpu(), "float32", tol32=2e-6 if dtype == "float32" else 1e-2)
+
+
 def attend(proj, d, dv, plan, scale=4.0, **form):
     Bk = B()
     n = proj.shape[0]
