@@ -6,7 +6,8 @@
 //                              queries to an fp32 buffer, keys and values into the cache entry of (request, position)
 //   paged_attention_kernel     one workgroup per (row tile, key/value head): up to 16 (token, query head) rows that share the
 //                              key/value head; key and value tiles of 64 positions are staged once in LDS (fp32) for all
-//                              rows; a wave owns up to four rows, a lane one key of the tile for the scores and value
+//                              rows; a wave owns up to four rows and takes them through a tile together (a key or value
+//                              read from LDS serves four products), a lane one key of the tile for the scores and value
 //                              columns lane, lane + 64, ... for the output; running maximum / sum per row.  Options
 //                              (AttnForm): keys restricted to the query's own run of `block` positions, a per-head sink
 //                              logit in the denominator, two softmax maps over the same values combined as
@@ -147,7 +148,10 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   float* s_k = sm;                                    // [64][qd + 1]
   float* s_v = s_k + kAttKeys * kd;                   // [64][vdim]
   float* s_q = s_v + kAttKeys * vdim;                 // [16][qd]
-  float* s_p = s_q + kAttRows * qd;                   // [4 waves][MAPS][64]
+  float* s_p = s_q + kAttRows * qd;                   // [4 waves][MAPS][64 keys][4 rows of the wave]
+  // 16-byte loads from the cache: every key / value row of the request starts at a multiple of eight values
+  const bool vec_k = (qd & 7) == 0 && (page_stride & 7) == 0 && (k_cache_off & 7) == 0 && aligned16(cache);
+  const bool vec_v = (vdim & 7) == 0 && (page_stride & 7) == 0 && (v_cache_off & 7) == 0 && aligned16(cache);
   const int tile = blockIdx.x, g = blockIdx.y;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int row0 = tile_row0[tile], ntok = tile_ntok[tile], qh0 = tile_qh0[tile], nqh = tile_nqh[tile];
@@ -182,51 +186,116 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   for (int k0 = kfirst + (int)blockIdx.z * kAttKeys; k0 < kmax; k0 += kAttKeys * nsplit) {
     const int nk = min(kAttKeys, kmax - k0);
     __syncthreads();
-    for (int i = tid; i < nk * qd; i += 256) {
-      const int j = i / qd, d = i % qd, p = k0 + j;
-      s_k[j * kd + d] = ld(cache + (int64_t)pages[p / page_size] * page_stride + k_cache_off + ((int64_t)(p % page_size) * G + g) * qd + d);
-    }
-    for (int i = tid; i < nk * vdim; i += 256) {
-      const int j = i / vdim, d = i % vdim, p = k0 + j;
-      s_v[j * vdim + d] = ld(cache + (int64_t)pages[p / page_size] * page_stride + v_cache_off + ((int64_t)(p % page_size) * G + g) * vdim + d);
+    {   // staging: four threads per key; one page lookup per thread and tile, 16-byte loads where the layout allows
+      const int j = tid >> 2, sub = tid & 3;
+      if (j < nk) {
+        const int p = k0 + j;
+        const int64_t pg = (int64_t)pages[p / page_size] * page_stride;
+        const A* kp = cache + pg + k_cache_off + ((int64_t)(p % page_size) * G + g) * qd;
+        const A* vp = cache + pg + v_cache_off + ((int64_t)(p % page_size) * G + g) * vdim;
+        float* dk = s_k + j * kd;
+        float* dv = s_v + j * vdim;
+        if (vec_k) {
+          for (int d = sub * 8; d < qd; d += 32) {
+            float t[8];
+            Vec8<A>::load(kp + d, t);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) dk[d + u] = t[u];
+          }
+        } else {
+          for (int d = sub; d < qd; d += 4) dk[d] = ld(kp + d);
+        }
+        if (vec_v) {
+          for (int d = sub * 8; d < vdim; d += 32) {
+            float t[8];
+            Vec8<A>::load(vp + d, t);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) dv[d + u] = t[u];
+          }
+        } else {
+          for (int d = sub; d < vdim; d += 4) dv[d] = ld(vp + d);
+        }
+      }
     }
     __syncthreads();
+    // the wave's (up to) four rows go through the tile together: a key value read from LDS serves four products
+    bool act[kAttRpw];
+    int jlo = nk, jhi = 0;
+    bool any = false;
 #pragma unroll
     for (int i = 0; i < kAttRpw; ++i) {
       const int lr = wave + 4 * i;
-      if (lr >= nrows) continue;                              // uniform over the wave
-      if (k0 > rpos[i] || k0 + nk <= rlo[i]) continue;        // the whole tile lies after this row's position or before its run
-      const bool seen = lane < nk && k0 + lane <= rpos[i] && k0 + lane >= rlo[i];
-      const int j0 = max(0, rlo[i] - k0), jn = min(nk, rpos[i] - k0 + 1);
+      // a row whose position lies before the tile, or whose run of visible keys begins after it, is left as it is
+      act[i] = lr < nrows && k0 <= rpos[i] && k0 + nk > rlo[i];
+      if (act[i]) {
+        any = true;
+        jlo = min(jlo, max(0, rlo[i] - k0));
+        jhi = max(jhi, min(nk, rpos[i] - k0 + 1));
+      }
+    }
+    if (!any) continue;       // uniform over the wave; the barriers are at the head of the loop, which every wave reaches
 #pragma unroll
-      for (int m = 0; m < MAPS; ++m) {
-        float s = -INFINITY;
-        if (seen) {
-          float a = 0.f;
-          const float* kr = s_k + lane * kd + m * dim;
-          const float* qr = s_q + lr * qd + m * dim;
-          for (int d = 0; d < dim; ++d) a = fmaf(qr[d], kr[d], a);
-          s = a * scale;
-        }
-        const float mnew = fmaxf(mrun[i][m], wave_max(s));
-        const float p = s == -INFINITY ? 0.f : expf(s - mnew);
-        const float corr = mrun[i][m] == -INFINITY ? 0.f : expf(mrun[i][m] - mnew);
-        lrun[i][m] = lrun[i][m] * corr + wave_sum(p);
-        mrun[i][m] = mnew;
-        float* pw = s_p + (wave * MAPS + m) * 64;
-        pw[lane] = p;
-        __builtin_amdgcn_wave_barrier();
+    for (int m = 0; m < MAPS; ++m) {
+      float a[kAttRpw] = {0.f, 0.f, 0.f, 0.f};
+      if (lane < nk) {
+        const float* kr = s_k + lane * kd + m * dim;
+        const float* qb = s_q + wave * qd + m * dim;        // row i of the wave: + 4 * i * qd
+        if ((dim & 3) == 0) {
+          for (int d = 0; d < dim; d += 4) {
+            const float k0v = kr[d], k1v = kr[d + 1], k2v = kr[d + 2], k3v = kr[d + 3];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int col = lane + 64 * c;
-          if (col < vdim) {
-            float a = acc[i][m][c] * corr;
-            for (int j = j0; j < jn; ++j) a = fmaf(pw[j], s_v[j * vdim + col], a);
-            acc[i][m][c] = a;
+            for (int i = 0; i < kAttRpw; ++i) {
+              const f32x4 qv = *reinterpret_cast<const f32x4*>(qb + 4 * i * qd + d);
+              a[i] = fmaf(qv.x, k0v, a[i]);
+              a[i] = fmaf(qv.y, k1v, a[i]);
+              a[i] = fmaf(qv.z, k2v, a[i]);
+              a[i] = fmaf(qv.w, k3v, a[i]);
+            }
+          }
+        } else {
+          for (int d = 0; d < dim; ++d) {
+            const float kv = kr[d];
+#pragma unroll
+            for (int i = 0; i < kAttRpw; ++i) a[i] = fmaf(qb[4 * i * qd + d], kv, a[i]);
           }
         }
-        __builtin_amdgcn_wave_barrier();
       }
+      float* pw = s_p + (wave * MAPS + m) * (64 * kAttRpw);   // [key][row of the wave]
+      float corr[kAttRpw];
+#pragma unroll
+      for (int i = 0; i < kAttRpw; ++i) {
+        corr[i] = 1.0f;
+        float pv = 0.f;
+        if (act[i]) {
+          const bool seen = lane < nk && k0 + lane <= rpos[i] && k0 + lane >= rlo[i];
+          const float sc = seen ? a[i] * scale : -INFINITY;
+          const float mnew = fmaxf(mrun[i][m], wave_max(sc));
+          pv = sc == -INFINITY ? 0.f : expf(sc - mnew);
+          corr[i] = mrun[i][m] == -INFINITY ? 0.f : expf(mrun[i][m] - mnew);
+          lrun[i][m] = lrun[i][m] * corr[i] + wave_sum(pv);
+          mrun[i][m] = mnew;
+        }
+        pw[lane * kAttRpw + i] = pv;
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int col = lane + 64 * c;
+        if (col < vdim) {
+          float o0 = act[0] ? acc[0][m][c] * corr[0] : acc[0][m][c], o1 = act[1] ? acc[1][m][c] * corr[1] : acc[1][m][c],
+                o2 = act[2] ? acc[2][m][c] * corr[2] : acc[2][m][c], o3 = act[3] ? acc[3][m][c] * corr[3] : acc[3][m][c];
+          for (int j = jlo; j < jhi; ++j) {    // weights outside a row's own range are exact zeros: they add nothing
+            const f32x4 pj = *reinterpret_cast<const f32x4*>(pw + j * kAttRpw);
+            const float v = s_v[j * vdim + col];
+            o0 = fmaf(pj.x, v, o0);
+            o1 = fmaf(pj.y, v, o1);
+            o2 = fmaf(pj.z, v, o2);
+            o3 = fmaf(pj.w, v, o3);
+          }
+          acc[0][m][c] = o0; acc[1][m][c] = o1; acc[2][m][c] = o2; acc[3][m][c] = o3;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
   }
   if (nsplit > 1) {   // [tile][kv head][split][row][map][vdim values | maximum | sum]
@@ -256,7 +325,8 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   }
 }
 
-// The states that the splits of a tile have left, folded in split order, then finished like an unsplit row.
+// The states that the splits of a tile have left, brought to their common maximum and summed in split order, then finished like
+// an unsplit row.
 template <typename A, int MAPS>
 __global__ __launch_bounds__(256) void paged_attention_merge_kernel(
     const float* __restrict__ part, int nsplit, int H, int G, int vdim, float factor, const int32_t* __restrict__ tile_row0,
@@ -267,26 +337,26 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(
   const int nrows = ntok * nqh, per_group = H / G;
   for (int lr = wave; lr < nrows; lr += 4) {
     float mrun[MAPS], lrun[MAPS], acc[MAPS][4];
+    const int64_t zs = (int64_t)kAttRows * MAPS * (vdim + 2);      // floats between two splits of a row
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
-      mrun[m] = -INFINITY;
-      lrun[m] = 0.f;
+      // lane z reads split z's maximum and sum; the common maximum and every split's weight follow without a dependent load,
+      // and the value loads of all splits are in flight together (nsplit <= 64)
+      const float* pr = part + ((((int64_t)(tile * G + g) * nsplit) * kAttRows + lr) * MAPS + m) * (vdim + 2);
+      const float mz = lane < nsplit ? pr[lane * zs + vdim] : -INFINITY;
+      const float lz = lane < nsplit ? pr[lane * zs + vdim + 1] : 0.f;
+      const float mall = wave_max(mz);
+      const float wz = mz == -INFINITY ? 0.f : expf(mz - mall);     // 0: a split that met no visible key
+      mrun[m] = mall;
+      lrun[m] = wave_sum(lz * wz);
 #pragma unroll
       for (int c = 0; c < 4; ++c) acc[m][c] = 0.f;
-    }
-    for (int z = 0; z < nsplit; ++z) {
-#pragma unroll
-      for (int m = 0; m < MAPS; ++m) {
-        const float* pr = part + ((((int64_t)(tile * G + g) * nsplit + z) * kAttRows + lr) * MAPS + m) * (vdim + 2);
-        const float mz = pr[vdim], lz = pr[vdim + 1];
-        if (mz == -INFINITY) continue;     // a split that met no visible key
-        const float mnew = fmaxf(mrun[m], mz);
-        const float c0 = mrun[m] == -INFINITY ? 0.f : expf(mrun[m] - mnew), c1 = expf(mz - mnew);
-        lrun[m] = lrun[m] * c0 + lz * c1;
-        mrun[m] = mnew;
+#pragma unroll 4
+      for (int z = 0; z < nsplit; ++z) {
+        const float w = __shfl(wz, z, kWave);
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-          if (lane + 64 * c < vdim) acc[m][c] = acc[m][c] * c0 + pr[lane + 64 * c] * c1;
+          if (lane + 64 * c < vdim) acc[m][c] = fmaf(pr[z * zs + lane + 64 * c], w, acc[m][c]);
       }
     }
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
@@ -360,12 +430,12 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
                                                 int32_t dtype, pegainfer_stream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_split < 1) n_split = 1;
-  if (n_split > 1 && (!workspace || n_split > 65535)) return PK_BAD;
+  if (n_split > 1 && (!workspace || n_split > 64)) return PK_BAD;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || (maps != 1 && maps != 2) || maps * dim > 256 || vdim <= 0 ||
       vdim > 256 || page_size <= 0 || kv_heads > 65535 || block < 0)
     return PK_BAD;
   const int qd = maps * dim;
-  const size_t smem = ((size_t)kAttKeys * (qd + 1) + (size_t)kAttKeys * vdim + (size_t)kAttRows * qd + 4 * maps * 64) * sizeof(float);
+  const size_t smem = ((size_t)kAttKeys * (qd + 1) + (size_t)kAttKeys * vdim + (size_t)kAttRows * qd + 4 * maps * 64 * kAttRpw) * sizeof(float);
   const dim3 grid(n_tiles, kv_heads, n_split);
   AttnForm form;
   form.block = block;
