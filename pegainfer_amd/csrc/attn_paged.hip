@@ -351,12 +351,19 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(
       lrun[m] = wave_sum(lz * wz);
 #pragma unroll
       for (int c = 0; c < 4; ++c) acc[m][c] = 0.f;
-#pragma unroll 4
-      for (int z = 0; z < nsplit; ++z) {
-        const float w = __shfl(wz, z, kWave);
+      for (int z0 = 0; z0 < nsplit; z0 += 8) {      // eight splits' values requested before the first is used
+        float val[8][4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-          if (lane + 64 * c < vdim) acc[m][c] = fmaf(pr[z * zs + lane + 64 * c], w, acc[m][c]);
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            val[u][c] = z0 + u < nsplit && lane + 64 * c < vdim ? pr[(z0 + u) * zs + lane + 64 * c] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const float w = __shfl(wz, min(z0 + u, 63), kWave);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) acc[m][c] = fmaf(val[u][c], w, acc[m][c]);
+        }
       }
     }
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;

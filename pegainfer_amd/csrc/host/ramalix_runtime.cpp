@@ -781,24 +781,16 @@ struct Model {
   }
   // out = Wdown (silu(Wgate in) * (Wup in))
   int swiglu(const void* gate_up, const void* down, int ff, const void* in, void* out, int T) {
-    if (linear(gate_up, in, gu, 2 * ff, T, D)) return -1;
-    RX_K(pegainfer_silu_mul_rows(gu, act, ff, T, dtype, S()));
+    // few rows (decoding) in bf16: the framework's GEMV with the SwiGLU in its epilogue, where its shapes allow
+    const bool fused = dtype == PEGAINFER_DTYPE_BF16 && !plain_kernels && T <= 16 && D % 8 == 0 &&
+                       pegainfer_gemv_fused(static_cast<const Half*>(gate_up), static_cast<const Half*>(in), static_cast<Half*>(act),
+                                            2 * ff, T, D, nullptr, nullptr, nullptr, eps, ff, S()) == 0;
+    if (!fused) {
+      if (linear(gate_up, in, gu, 2 * ff, T, D)) return -1;
+      RX_K(pegainfer_silu_mul_rows(gu, act, ff, T, dtype, S()));
+    }
     return linear(down, act, out, D, T, ff);
   }
-  // hb = n32 + time_conv(n32), then the tail of the (run, request) moves on
-  int input_conv(const void* w, int64_t st_off, int64_t slot_stride, bool single, int n, int T, const int32_t* d_ent,
-                 const int32_t* d_row0, const int32_t* d_slot) {
-    if (single) {
-      RX_K(pegainfer_time_conv_step(n32, PEGAINFER_DTYPE_F32, D, w, dtype, state + st_off, slot_stride, hb, dtype, D, D, canon_taps, 1,
-                                    d_slot, n, S()));
-    } else {
-      RX_K(pegainfer_time_conv(n32, PEGAINFER_DTYPE_F32, D, w, dtype, state + st_off, slot_stride, hb, dtype, D, D, canon_taps, 1, d_ent,
-                               d_row0, d_slot, T, S()));
-      RX_K(pegainfer_time_conv_commit(n32, PEGAINFER_DTYPE_F32, D, state + st_off, slot_stride, D, canon_taps, d_row0, d_slot, n, S()));
-    }
-    return 0;
-  }
-
   int step(int n, const int32_t* ids, const int32_t* lens, const uint32_t* tokens, int n_want, const int32_t* want_rows,
            float* out_logits, int32_t* out_tokens) {
     if (!finalized) return set_error("step before finalize");
@@ -931,6 +923,26 @@ struct Model {
     }
     // ---- the layer runs (everything below reads the step's shape from its arguments and the step's contents from the
     //      metadata block, so a launch sequence recorded for one decode step serves every later step of the same shape)
+    // x <- x + mlt (yv + bias) + add_rows + add_vec; with a gain also the norm of the sublayer that follows and its input
+    // convolution (hb = n + conv(n), the tail moved on)
+    auto open_sublayer = [&](const void* yv, const void* bias, float mlt, const float* add_rows, const void* add_vec, bool write_x,
+                             const void* gain, const void* conv_w, int64_t st_off) -> int {
+      if (!gain) {
+        RX_K(pegainfer_scalar_rms_add(x, yv, dtype, bias, mlt, add_rows, add_vec, x, nullptr, eps, nullptr, D, Ti, dtype, S()));
+        return 0;
+      }
+      RX_K(pegainfer_scalar_rms_add(x, yv, dtype, bias, mlt, add_rows, add_vec, write_x ? x : nullptr, gain, eps, n32, D, Ti, dtype, S()));
+      if (single) {   // output and the moved-on tail in one launch (folding it into the norm's launch was measured: one workgroup
+                      // per row then walks every channel's tail, 15 us against 5.6 + 4.3)
+        RX_K(pegainfer_time_conv_step(n32, PEGAINFER_DTYPE_F32, D, conv_w, dtype, state + st_off, slot_stride, hb, dtype, D, D,
+                                      canon_taps, 1, d_slot, n, S()));
+        return 0;
+      }
+      RX_K(pegainfer_time_conv(n32, PEGAINFER_DTYPE_F32, D, conv_w, dtype, state + st_off, slot_stride, hb, dtype, D, D, canon_taps, 1,
+                               d_ent, d_row0, d_slot, Ti, S()));
+      RX_K(pegainfer_time_conv_commit(n32, PEGAINFER_DTYPE_F32, D, state + st_off, slot_stride, D, canon_taps, d_row0, d_slot, n, S()));
+      return 0;
+    };
     auto run_layers = [&]() -> int {
     RX_K(pegainfer_embed_f32(embed, d_tok, emb, D, Ti, dtype, S()));
     RX_K(pegainfer_embed_f32(embed, d_tok, x, D, Ti, dtype, S()));
@@ -941,13 +953,13 @@ struct Model {
       const int Mp = c.proj_rows;
       if (r.pass >= 0) {
         // a pass over the repeated span begins: the embedding rows again (not before the first pass), this pass's own row,
-        // and the norm of the first sublayer in the same launch
-        RX_K(pegainfer_scalar_rms_add(x, nullptr, dtype, nullptr, 0.f, r.pass > 0 ? emb : nullptr,
-                                      at(loop_step, (size_t)r.pass * D), x, w.norm1, eps, n32, D, Ti, dtype, S()));
+        // and the first sublayer's norm and input convolution
+        if (open_sublayer(nullptr, nullptr, 0.f, r.pass > 0 ? emb : nullptr, at(loop_step, (size_t)r.pass * D), true, w.norm1, w.canon1,
+                          r.st_canon1))
+          return -1;
       } else if (ri == 0) {
-        RX_K(pegainfer_scalar_rms_add(x, nullptr, dtype, nullptr, 0.f, nullptr, nullptr, nullptr, w.norm1, eps, n32, D, Ti, dtype, S()));
-      }   // otherwise the launch that closed the run before has left n32
-      if (input_conv(w.canon1, r.st_canon1, slot_stride, single, n, Ti, d_ent, d_row0, d_slot)) return -1;
+        if (open_sublayer(nullptr, nullptr, 0.f, nullptr, nullptr, false, w.norm1, w.canon1, r.st_canon1)) return -1;
+      }   // otherwise the launch that closed the run before has left hb
       if (linear(w.proj, hb, proj, Mp, Ti, D)) return -1;
       if (c.type == kChannelDelta) {
         const DeltaCfg& d = c.dl;
@@ -989,16 +1001,14 @@ struct Model {
       // what the launch that closes this run norms for: the next run's first sublayer, unless that run opens a pass (its own
       // launch sums first) or there is none (the final norm runs on the wanted rows only)
       const bool next_plain = ri + 1 < runs.size() && runs[ri + 1].pass < 0;
-      const void* next_gain = next_plain ? weights[(size_t)runs[ri + 1].layer].norm1 : nullptr;
+      const LayerW* nw = next_plain ? &weights[(size_t)runs[ri + 1].layer] : nullptr;
+      const int64_t next_st = next_plain ? runs[ri + 1].st_canon1 : 0;
       if (c.mlp.kind) {
-        RX_K(pegainfer_scalar_rms_add(x, y, dtype, w.o_bias, mult, nullptr, nullptr, x, w.norm2, eps, n32, D, Ti, dtype, S()));
-        if (input_conv(w.canon2, r.st_canon2, slot_stride, single, n, Ti, d_ent, d_row0, d_slot)) return -1;
+        if (open_sublayer(y, w.o_bias, mult, nullptr, nullptr, true, w.norm2, w.canon2, r.st_canon2)) return -1;
         if (routed_ff(c, w, Ti)) return -1;
-        RX_K(pegainfer_scalar_rms_add(x, y, dtype, nullptr, mult, nullptr, nullptr, x, next_gain, eps, next_gain ? n32 : nullptr, D, Ti,
-                                      dtype, S()));
-      } else {
-        RX_K(pegainfer_scalar_rms_add(x, y, dtype, w.o_bias, mult, nullptr, nullptr, x, next_gain, eps, next_gain ? n32 : nullptr, D, Ti,
-                                      dtype, S()));
+        if (open_sublayer(y, nullptr, mult, nullptr, nullptr, true, nw ? nw->norm1 : nullptr, nw ? nw->canon1 : nullptr, next_st)) return -1;
+      } else if (open_sublayer(y, w.o_bias, mult, nullptr, nullptr, true, nw ? nw->norm1 : nullptr, nw ? nw->canon1 : nullptr, next_st)) {
+        return -1;
       }
       if (tap_on) RX_HIP(hipMemcpyAsync(tap + ri * T * D, x, T * D * 4, hipMemcpyDeviceToDevice, stream));
     }
