@@ -304,7 +304,10 @@ pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, 
  * scale, key or value.  head_norm != 0: out / sqrt(mean(out^2) + norm_eps) over the head's vdim values.  `factor` comes last.
  * n_split > 1: every tile's keys are dealt in tiles of 64 to n_split workgroups (split z takes key tiles z, z + n_split, ...:
  * the grid does not depend on the contexts' lengths) whose softmax states a second launch folds in split order - for steps of
- * few rows over long contexts (decoding); `workspace` then holds pegainfer_paged_attention_workspace(...) floats. */
+ * few rows over long contexts (decoding); `workspace` then holds pegainfer_paged_attention_workspace(...) floats.
+ * Two kernels behind the entry: a bf16 cache runs on the matrix cores (q and the softmax weights rounded to bf16 where they enter
+ * them; scores, maxima, sums and outputs fp32) unless plain != 0; an fp32 cache, or plain, runs the fp32-FMA kernel.
+ * pegainfer_paged_attention is the plain kernel's plain form. */
 pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
                                                 int64_t v_cache_off, int32_t page_size, const int32_t* positions,
                                                 const int32_t* row_entry, const int32_t* page_indptr, const int32_t* page_ids,
@@ -313,7 +316,7 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
                                                 const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
                                                 int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
                                                 int32_t head_norm, float norm_eps, int32_t n_split, float* workspace,
-                                                int32_t dtype, pegainfer_stream_t stream);
+                                                int32_t plain, int32_t dtype, pegainfer_stream_t stream);
 /* fp32 values of scratch a launch with n_split > 1 needs (0 for n_split <= 1) */
 int64_t pegainfer_paged_attention_workspace(int32_t n_tiles, int32_t kv_heads, int32_t vdim, int32_t maps, int32_t n_split);
 /* out[row, :cols] = in[row, :cols] * factor; rows of in / out at their own strides (elements of dtype) */

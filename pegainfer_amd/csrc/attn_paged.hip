@@ -325,6 +325,237 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   }
 }
 
+// The same attention on the matrix cores, for a bf16 cache (v_mfma_f32_16x16x16_bf16 for both products).  Same tiles: up to 16
+// (token, query head) rows of one key/value head per workgroup, key tiles of 64 positions on the grid that starts at position 0.
+// Each of the four waves owns 16 keys of a tile and is a softmax stream of its own over them (its own running maximum, sum and
+// output block for all 16 rows), so a tile costs no exchange between waves; the four streams are folded once, after the last
+// tile, through LDS.  A wave computes S^T = K Q^T: the result leaves lane l with the scores of row l % 16 against keys
+// 4 (l / 16) .. + 3 - exactly the A operand (weights, rounded to bf16) the second product P V wants from it; its B operand comes
+// from a transposed copy of the value tile in LDS.  Scores, maxima, sums and outputs are fp32; q and the weights are rounded to
+// bf16 where they enter the matrix cores, and the row sum is taken over the rounded weights.  dim is padded to a multiple of
+// 16 per map, vdim to NCB * 16 columns (zeros).
+typedef short v4s_t __attribute__((ext_vector_type(4)));
+constexpr int kMfVs = kAttKeys + 4;     // row stride of the transposed value tile (bf16 values; 8-byte aligned rows)
+
+template <int MAPS, int NCB>
+__global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
+    const float* __restrict__ q, const uint16_t* __restrict__ cache, int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
+    int page_size, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_entry,
+    const int32_t* __restrict__ page_indptr, const int32_t* __restrict__ page_ids, int H, int G, int dim, int vdim, float scale,
+    float factor, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ tile_ntok,
+    const int32_t* __restrict__ tile_qh0, const int32_t* __restrict__ tile_nqh, uint16_t* __restrict__ out, int64_t out_stride,
+    AttnForm form, int nsplit, float* __restrict__ part) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
+  constexpr int VP = NCB * 16;
+  const int qd = MAPS * dim, dp = (dim + 15) & ~15, ks = MAPS * dp + 4;
+  uint16_t* s_k = reinterpret_cast<uint16_t*>(smraw);        // [64][ks]
+  uint16_t* s_q = s_k + kAttKeys * ks;                         // [16][ks]
+  uint16_t* s_vt = s_q + kAttRows * ks;                        // [VP][kMfVs]: value column major
+  float* f_buf = reinterpret_cast<float*>(smraw);              // after the last tile: [2][MAPS][16][VP] partial outputs,
+  float* f_st = f_buf + 2 * MAPS * kAttRows * VP;              //   [4 waves][MAPS][16][2] maxima and sums, [MAPS][16][2] folded
+  float* f_fin = f_st + 4 * MAPS * kAttRows * 2;
+  const int tile = blockIdx.x, g = blockIdx.y;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lrow = lane & 15, lgrp = lane >> 4;
+  const int row0 = tile_row0[tile], ntok = tile_ntok[tile], qh0 = tile_qh0[tile], nqh = tile_nqh[tile];
+  const int nrows = ntok * nqh, per_group = H / G;
+  const int e = row_entry[row0];
+  const int32_t* pages = page_ids + page_indptr[e];
+  const int kmax = positions[row0 + ntok - 1] + 1;
+  const int kfirst = form.block > 0 ? ((positions[row0] / form.block) * form.block / kAttKeys) * kAttKeys : 0;
+  // zeros everywhere first: padding columns, rows past the tile's, keys past the context's end must multiply as zeros
+  for (int i = tid; i < (kAttKeys + kAttRows) * ks + VP * kMfVs; i += 256) s_k[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < nrows * qd; i += 256) {
+    const int lr = i / qd, c = i % qd;
+    const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
+    s_q[lr * ks + (c / dim) * dp + c % dim] = f2bf(q[((int64_t)(row0 + tok) * H + qh) * qd + c]);
+  }
+  const int rpos = lrow < nrows ? positions[row0 + lrow / nqh] : -1;      // this lane's row (as a column of S^T)
+  const int rlo = form.block > 0 && rpos >= 0 ? (rpos / form.block) * form.block : 0;
+  float mrun[MAPS], lrun[MAPS];
+  f32x4 o[MAPS][NCB];
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) {
+    mrun[m] = -INFINITY;
+    lrun[m] = 0.f;
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) o[m][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const bool vec_k = (dim & 7) == 0 && (page_stride & 7) == 0 && (k_cache_off & 7) == 0 && aligned16(cache);
+  const bool vec_v = (vdim & 7) == 0 && (page_stride & 7) == 0 && (v_cache_off & 7) == 0 && aligned16(cache);
+  for (int k0 = kfirst + (int)blockIdx.z * kAttKeys; k0 < kmax; k0 += kAttKeys * nsplit) {
+    const int nk = min(kAttKeys, kmax - k0);
+    __syncthreads();
+    {   // staging: four threads per key; the value tile is written transposed
+      const int j = tid >> 2, sub = tid & 3;
+      if (j < nk) {
+        const int p = k0 + j;
+        const int64_t pg = (int64_t)pages[p / page_size] * page_stride;
+        const uint16_t* kp = cache + pg + k_cache_off + ((int64_t)(p % page_size) * G + g) * qd;
+        const uint16_t* vp = cache + pg + v_cache_off + ((int64_t)(p % page_size) * G + g) * vdim;
+        uint16_t* dk = s_k + j * ks;
+        if (vec_k) {
+          for (int c = sub * 8; c < qd; c += 32) {
+            const u32x4 t = *reinterpret_cast<const u32x4*>(kp + c);
+            uint16_t* dst = dk + (c / dim) * dp + c % dim;           // 8-byte aligned (ks * 2 is a multiple of 8 only)
+            *reinterpret_cast<u32x2*>(dst) = u32x2{t.x, t.y};
+            *reinterpret_cast<u32x2*>(dst + 4) = u32x2{t.z, t.w};
+          }
+        } else {
+          for (int c = sub; c < qd; c += 4) dk[(c / dim) * dp + c % dim] = kp[c];
+        }
+        if (vec_v) {
+          for (int c = sub * 8; c < vdim; c += 32) {
+            const u32x4 t = *reinterpret_cast<const u32x4*>(vp + c);
+            const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              s_vt[(c + 2 * u) * kMfVs + j] = (uint16_t)(w[u] & 0xFFFFu);
+              s_vt[(c + 2 * u + 1) * kMfVs + j] = (uint16_t)(w[u] >> 16);
+            }
+          }
+        } else {
+          for (int c = sub; c < vdim; c += 4) s_vt[c * kMfVs + j] = vp[c];
+        }
+      }
+    }
+    __syncthreads();
+    const int kb = wave * 16;                       // this wave's keys of the tile
+    if (k0 + kb >= kmax) continue;                  // uniform over the wave; barriers sit at the loop's head
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
+      const uint16_t* ka = s_k + (kb + lrow) * ks + m * dp + 4 * lgrp;
+      const uint16_t* qb = s_q + lrow * ks + m * dp + 4 * lgrp;
+      for (int kk = 0; kk < dp; kk += 16)
+        sc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const v4s_t*>(ka + kk), *reinterpret_cast<const v4s_t*>(qb + kk),
+                                                       sc, 0, 0, 0);
+      float sv[4] = {sc.x, sc.y, sc.z, sc.w};
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kp_ = k0 + kb + 4 * lgrp + r;
+        sv[r] = (kp_ <= rpos && kp_ >= rlo) ? sv[r] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sv[r]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float mnew = fmaxf(mrun[m], tmax);
+      const float corr = mnew == -INFINITY ? 1.0f : (mrun[m] == -INFINITY ? 0.f : expf(mrun[m] - mnew));
+      uint16_t pb[4];
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pb[r] = f2bf(sv[r] == -INFINITY ? 0.f : expf(sv[r] - mnew));
+        psum += bf2f(pb[r]);
+      }
+      psum += __shfl_xor(psum, 16, kWave);
+      psum += __shfl_xor(psum, 32, kWave);
+      lrun[m] = lrun[m] * corr + psum;
+      mrun[m] = mnew;
+      // the output block holds rows 4 (l / 16) + r: their factors sit in the lanes of those numbers
+      float cr[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, 4 * lgrp + r, kWave);
+      v4s_t pa;
+      pa.x = (short)pb[0]; pa.y = (short)pb[1]; pa.z = (short)pb[2]; pa.w = (short)pb[3];
+      const uint16_t* vb = s_vt + lrow * kMfVs + kb + 4 * lgrp;
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) {
+        f32x4 t = o[m][cb];
+        t.x *= cr[0]; t.y *= cr[1]; t.z *= cr[2]; t.w *= cr[3];
+        o[m][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa, *reinterpret_cast<const v4s_t*>(vb + cb * 16 * kMfVs), t, 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();                                  // the tiles' LDS is free: the four streams are folded through it
+  if (lane < 16) {
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      f_st[((wave * MAPS + m) * kAttRows + lane) * 2] = mrun[m];
+      f_st[((wave * MAPS + m) * kAttRows + lane) * 2 + 1] = lrun[m];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) {
+    float mall = -INFINITY, lall = 0.f, mine = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mall = fmaxf(mall, f_st[((w * MAPS + m) * kAttRows + lrow) * 2]);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = f_st[((w * MAPS + m) * kAttRows + lrow) * 2];
+      const float sw = mw == -INFINITY ? 0.f : expf(mw - mall);
+      lall += f_st[((w * MAPS + m) * kAttRows + lrow) * 2 + 1] * sw;
+      if (w == wave) mine = sw;
+    }
+    if (wave == 0 && lane < 16) {
+      f_fin[(m * kAttRows + lane) * 2] = mall;
+      f_fin[(m * kAttRows + lane) * 2 + 1] = lall;
+    }
+    float cr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cr[r] = __shfl(mine, 4 * lgrp + r, kWave);
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) { o[m][cb].x *= cr[0]; o[m][cb].y *= cr[1]; o[m][cb].z *= cr[2]; o[m][cb].w *= cr[3]; }
+  }
+  // element (map m, row 4 (l / 16) + r, column 16 cb + l % 16) of a wave's block
+  auto slot = [&](int b, int m, int cb, int r) { return f_buf + ((b * MAPS + m) * kAttRows + 4 * lgrp + r) * VP + cb * 16 + lrow; };
+  auto put = [&](int b) {
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) { *slot(b, m, cb, 0) = o[m][cb].x; *slot(b, m, cb, 1) = o[m][cb].y; *slot(b, m, cb, 2) = o[m][cb].z; *slot(b, m, cb, 3) = o[m][cb].w; }
+  };
+  auto take = [&](int b) {
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) { o[m][cb].x += *slot(b, m, cb, 0); o[m][cb].y += *slot(b, m, cb, 1); o[m][cb].z += *slot(b, m, cb, 2); o[m][cb].w += *slot(b, m, cb, 3); }
+  };
+  if (wave >= 2) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) take(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave == 0) { take(0); put(0); }
+  __syncthreads();
+  // rows go back to the layout of the plain kernel: wave w finishes rows w, w + 4, ...; a lane holds columns l, l + 64, ...
+  float* pbase = nsplit > 1 ? part + (((int64_t)(tile * G + g) * nsplit + blockIdx.z) * kAttRows) * MAPS * (vdim + 2) : nullptr;
+  for (int lr = wave; lr < nrows; lr += 4) {
+    float fm[MAPS], fl[MAPS], acc[MAPS][4];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      fm[m] = f_fin[(m * kAttRows + lr) * 2];
+      fl[m] = f_fin[(m * kAttRows + lr) * 2 + 1];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[m][c] = lane + 64 * c < vdim ? f_buf[(m * kAttRows + lr) * VP + lane + 64 * c] : 0.f;
+    }
+    if (nsplit > 1) {
+#pragma unroll
+      for (int m = 0; m < MAPS; ++m) {
+        float* pr = pbase + ((int64_t)lr * MAPS + m) * (vdim + 2);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (lane + 64 * c < vdim) pr[lane + 64 * c] = acc[m][c];
+        if (lane == 0) { pr[vdim] = fm[m]; pr[vdim + 1] = fl[m]; }
+      }
+      continue;
+    }
+    const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
+    attn_finish_row<uint16_t, MAPS>(fm, fl, acc, form, qh, vdim, factor, lane, out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
+  }
+}
+
+// bytes of LDS the matrix-core kernel needs: the tiles while the keys are walked, the fold buffers afterwards
+static size_t mfma_attention_lds(int maps, int dim, int ncb) {
+  const size_t ks = (size_t)maps * ((dim + 15) & ~15) + 4, vp = (size_t)ncb * 16;
+  const size_t tiles = ((kAttKeys + kAttRows) * ks + vp * kMfVs) * sizeof(uint16_t);
+  const size_t fold = (2 * maps * kAttRows * vp + 4 * maps * kAttRows * 2 + maps * kAttRows * 2) * sizeof(float);
+  return std::max(tiles, fold);
+}
+
 // The states that the splits of a tile have left, brought to their common maximum and summed in split order, then finished like
 // an unsplit row.
 template <typename A, int MAPS>
@@ -434,7 +665,7 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
                                                 const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
                                                 int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
                                                 int32_t head_norm, float norm_eps, int32_t n_split, float* workspace,
-                                                int32_t dtype, pegainfer_stream_t stream) {
+                                                int32_t plain, int32_t dtype, pegainfer_stream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_split < 1) n_split = 1;
   if (n_split > 1 && (!workspace || n_split > 64)) return PK_BAD;
@@ -451,6 +682,39 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
   form.head_norm = head_norm;
   form.norm_eps = norm_eps;
   bool ok = true;
+  if (dtype == kDtBf16 && !plain) {   // bf16 cache: the matrix-core kernel; same tiles, same splits, same merge
+    const int ncb = vdim <= 32 ? 2 : vdim <= 64 ? 4 : vdim <= 128 ? 8 : 16;
+    const size_t lds = mfma_attention_lds(maps, dim, ncb);
+    auto launch = [&](auto kern) {
+      if (lds > 48 * 1024 &&
+          hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        ok = false;
+        return;
+      }
+      kern<<<grid, 256, lds, as_stream(stream)>>>(q, static_cast<const uint16_t*>(cache), page_stride, k_cache_off, v_cache_off, page_size,
+                                                  positions, row_entry, page_indptr, page_ids, heads, kv_heads, dim, vdim, scale, factor,
+                                                  tile_row0, tile_ntok, tile_qh0, tile_nqh, static_cast<uint16_t*>(out), out_stride, form,
+                                                  n_split, workspace);
+    };
+    auto by_cols = [&](auto maps_c) {
+      constexpr int M = decltype(maps_c)::value;
+      if (ncb == 2) launch(paged_attention_mfma_kernel<M, 2>);
+      else if (ncb == 4) launch(paged_attention_mfma_kernel<M, 4>);
+      else if (ncb == 8) launch(paged_attention_mfma_kernel<M, 8>);
+      else launch(paged_attention_mfma_kernel<M, 16>);
+    };
+    if (maps == 1) by_cols(std::integral_constant<int, 1>());
+    else by_cols(std::integral_constant<int, 2>());
+    if (ok && n_split > 1) {
+      if (maps == 1)
+        paged_attention_merge_kernel<uint16_t, 1><<<dim3(n_tiles, kv_heads), 256, 0, as_stream(stream)>>>(
+            workspace, n_split, heads, kv_heads, vdim, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh, static_cast<uint16_t*>(out), out_stride, form);
+      else
+        paged_attention_merge_kernel<uint16_t, 2><<<dim3(n_tiles, kv_heads), 256, 0, as_stream(stream)>>>(
+            workspace, n_split, heads, kv_heads, vdim, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh, static_cast<uint16_t*>(out), out_stride, form);
+    }
+    return ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
+  }
   const bool known = by_dtype(dtype, [&](auto* t) {
     using A = std::remove_pointer_t<decltype(t)>;
     auto go = [&](auto kern) {
@@ -492,7 +756,7 @@ pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, 
                                              int64_t out_stride, int32_t dtype, pegainfer_stream_t stream) {
   return pegainfer_paged_attention_ex(q, cache, page_stride, k_cache_off, v_cache_off, page_size, positions, row_entry, page_indptr,
                                       page_ids, heads, kv_heads, dim, vdim, scale, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh,
-                                      n_tiles, out, out_stride, 1, 0.f, 0, nullptr, 0, 0.f, 1, nullptr, dtype, stream);
+                                      n_tiles, out, out_stride, 1, 0.f, 0, nullptr, 0, 0.f, 1, nullptr, 1, dtype, stream);
 }
 
 pegainfer_status_t pegainfer_scale_rows(const void* in, int64_t in_stride, void* out, int64_t out_stride, int32_t cols,

@@ -995,7 +995,7 @@ struct Model {
         RX_K(pegainfer_paged_attention_ex(q32, cache, page_stride, r.k_off, r.v_off, kPageSize, d_pos, d_ent, d_ind, d_pages, a.heads,
                                           a.kv, a.dim, a.vdim, a.scale, two ? 1.0f - a.diff : 1.0f, tb, tb + tile_cnt[ts],
                                           tb + 2 * tile_cnt[ts], tb + 3 * tile_cnt[ts], (int)tile_cnt[ts], mix, c.mix_cols, a.maps,
-                                          w.lambda, a.block, w.sink, two ? 1 : 0, eps, nsplit, att_part, dtype, S()));
+                                          w.lambda, a.block, w.sink, two ? 1 : 0, eps, nsplit, att_part, plain_kernels ? 1 : 0, dtype, S()));
       }
       if (linear(w.o, mix, y, D, Ti, c.mix_cols)) return -1;
       // what the launch that closes this run norms for: the next run's first sublayer, unless that run opens a pass (its own

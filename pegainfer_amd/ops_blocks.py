@@ -347,8 +347,9 @@ def qk_prep_paged(proj, offs, heads, kv_heads, dim, vdim, rg, page_indptr, page_
 
 
 def paged_attention_ex(q, cache, page_stride, k_off, v_off, page_size, rg, page_indptr, page_ids, kv_heads, vdim, scale, factor=1.0,
-                       maps=1, lam=0.0, block=0, sink=None, head_norm=False, norm_eps=0.0, n_split=1):
-    """q fp32 [rows, heads, maps * dim]; n_split > 1: the keys of every tile dealt to that many workgroups, then merged"""
+                       maps=1, lam=0.0, block=0, sink=None, head_norm=False, norm_eps=0.0, n_split=1, plain=False):
+    """q fp32 [rows, heads, maps * dim]; n_split > 1: the keys of every tile dealt to that many workgroups, then merged; a bf16 cache runs on
+    the matrix cores unless plain"""
     T, H, qd = q.shape
     out = torch.empty((T, H * vdim), dtype=cache.dtype, device=q.device)
     t = attention_tiles(rg.lens, H // kv_heads, q.device)
@@ -360,7 +361,7 @@ def paged_attention_ex(q, cache, page_stride, k_off, v_off, page_size, rg, page_
                                                 _p(rg.row_entry), _p(page_indptr), _p(page_ids), H, kv_heads, qd // maps, vdim,
                                                 float(scale), float(factor), _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), t[0].numel(),
                                                 _p(out), out.stride(0), maps, float(lam), int(block), _p(sink), int(bool(head_norm)),
-                                                float(norm_eps), int(n_split), _p(ws), _dt(cache), _stream()), "paged_attention_ex")
+                                                float(norm_eps), int(n_split), _p(ws), int(bool(plain)), _dt(cache), _stream()), "paged_attention_ex")
     return out
 
 

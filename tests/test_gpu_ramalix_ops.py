@@ -190,6 +190,9 @@ def test_key_splits_agree_with_the_unsplit_launch(dtype, n_split):
             whole = Bk.paged_attention_ex(*args, **form)
             cut = Bk.paged_attention_ex(*args, n_split=n_split, **form)
             close(cut, whole.double().cpu(), "float32", tol32=2e-6 if dtype == "float32" else 1e-2)
+            if dtype == "bfloat16":      # the matrix-core kernel (the default for a bf16 cache) against the fp32-FMA kernel
+                close(Bk.paged_attention_ex(*args, plain=True, **form), whole.double().cpu(), "float32", tol32=2e-2)
+                close(Bk.paged_attention_ex(*args, plain=True, n_split=n_split, **form), whole.double().cpu(), "float32", tol32=2e-2)
 
 
 def attend(proj, d, dv, plan, scale=4.0, **form):
