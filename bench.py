@@ -671,6 +671,8 @@ def main():
     ap.add_argument("--fz-only", default="both", choices=["both", "feruzen", "qwen35"], help="--model feruzen: which side to run")
     ap.add_argument("--rx-size", default="mid", choices=["small", "mid", "large", "all"], help="layer sizes of --model ramalix")
     ap.add_argument("--rx-only", default="both", choices=["both", "ramalix", "feruzen"], help="--model ramalix: which side to run")
+    ap.add_argument("--rx-phase", default="all", choices=["all", "prefill", "decode"],
+                    help="--model ramalix: prefill or decode (bs 1) alone, for a kernel trace of that phase")
     ap.add_argument("--decode-mode", type=int, choices=[0, 1], default=int(os.environ.get("PEGAINFER_DECODE_MODE", "1")),
                     help="0 = reference op sequence 1:1, 1 = fused MI355X decode kernels (bit-identical)")
     ap.add_argument("--split-policy", type=int, default=1)

@@ -32,12 +32,13 @@ def ramalix_config(s):
 
 
 def feruzen_config(s):
-    """the same layer runs as eight Feruzen layers: attention layers with 128-wide heads (beside a matrix memory as small as
-    the design allows), delta layers of equal heads, the same experts on every layer"""
+    """the same layer runs as eight Feruzen layers: attention layers with 128-wide heads (beside one small matrix memory head,
+    which that design's attention layers cannot go without; 128 values wide so that the joint output projection keeps a width
+    the tuned GEMM routes take), delta layers of equal heads, the same experts on every layer"""
     moe = {"kind": "moe", "expert": {"ff": s["eff"], "limit": 7.0}, "router": {"experts": s["experts"], "top": s["top"]},
            "shared": {"ff": s["sff"], "limit": 7.0}}
     par = {"left": {"heads": s["heads"], "kv_heads": s["kv"], "dim": 128, "vdim": 128, "rot": {"base": 1e6, "dims": 64}, "scale": 128 ** -0.5},
-           "right": {"heads": 1, "dim": 16, "vdim": 16, "gate_cap": 15.0}, "left_scale": 1.0, "right_scale": 1.0}
+           "right": {"heads": 1, "dim": 16, "vdim": 128, "gate_cap": 15.0}, "left_scale": 1.0, "right_scale": 1.0}
     dl = {"heads": s["lin_v"], "kv_heads": s["lin_k"], "dim": 128, "vdim": 128, "conv": 4}
     four = [{"type": "parallel", "mixer": par, "mlp": moe}, {"type": "parallel", "mixer": par, "mlp": moe},
             {"type": "delta", "mixer": dl, "mlp": moe}, {"type": "parallel", "mixer": par, "mlp": moe}]
@@ -53,7 +54,7 @@ def _timed(fn, iters):
     return (time.perf_counter() - t0) / iters
 
 
-def measure(engine_cls, cfg, s, prompt_len, ctx, batches, iters):
+def measure(engine_cls, cfg, s, prompt_len, ctx, batches, iters, phase="all"):
     eng = engine_cls(cfg, max_tokens=max(batches) * (ctx + 64) + prompt_len + 64, max_requests=max(batches),
                      dtype="bfloat16").fill_synthetic(seed=1, std=0.02)
     prompt = [(100 + i) % s["vocab"] for i in range(prompt_len)]
@@ -63,9 +64,10 @@ def measure(engine_cls, cfg, s, prompt_len, ctx, batches, iters):
         r = eng.new_request()
         eng.step([(r, prompt)], logits=False, tokens=True)
         eng.drop_request(r)
-    out["prefill_tok_s"] = round(prompt_len / _timed(prefill, iters), 1)
-    out["prefill_device_ms"] = round(eng.last_step_ms(), 3)
-    for bs in batches:
+    if phase in ("all", "prefill"):
+        out["prefill_tok_s"] = round(prompt_len / _timed(prefill, iters), 1)
+        out["prefill_device_ms"] = round(eng.last_step_ms(), 3)
+    for bs in batches if phase in ("all", "decode") else ():
         rids = [eng.new_request() for _ in range(bs)]
         eng.step([(r, prompt[:ctx]) for r in rids], logits=False, tokens=True)
         dt = _timed(lambda: eng.step([(r, [7]) for r in rids], logits=False, tokens=True), max(iters, 20))
@@ -82,14 +84,16 @@ def run(args):
     from .ramalix import RamalixEngine
     sizes = [args.rx_size] if args.rx_size != "all" else list(SIZES)
     which = getattr(args, "rx_only", "both")
+    phase = getattr(args, "rx_phase", "all")        # one phase alone gives a kernel trace of that phase only
+    batches = (1, 4) if phase == "all" else (1,)
     res = {}
     for name in sizes:
         s = SIZES[name]
         res[name] = {"layer_runs": RUNS, "sizes": s}
         if which in ("both", "ramalix"):
-            res[name]["ramalix"] = measure(RamalixEngine, ramalix_config(s), s, args.ctx, args.ctx, (1, 4), max(2, args.warmup))
+            res[name]["ramalix"] = measure(RamalixEngine, ramalix_config(s), s, args.ctx, args.ctx, batches, max(2, args.warmup), phase)
         if which in ("both", "feruzen"):
-            res[name]["feruzen_equal_size"] = measure(FeruzenEngine, feruzen_config(s), s, args.ctx, args.ctx, (1, 4), max(2, args.warmup))
+            res[name]["feruzen_equal_size"] = measure(FeruzenEngine, feruzen_config(s), s, args.ctx, args.ctx, batches, max(2, args.warmup), phase)
     print(json.dumps({"metric": "ramalix_vs_feruzen_layer_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
                       "n_gpus": 1, "prompt_len": args.ctx, "decode_ctx": args.ctx, "results": res}))
     return 0
