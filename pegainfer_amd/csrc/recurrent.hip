@@ -132,12 +132,21 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     S[i] = d < dim && col < vdim ? S_g[(int64_t)d * vdim + col] : 0.f;
   }
   RoundFetch<NS> nxt;
+  float gnx[CH ? NS : 1];     // the next round's channel decays, fetched with its q | k | v (same thread-to-value map)
   auto fetch = [&](int t0) {
     const float* base = qkv + (int64_t)(row0 + t0) * qkv_stride;
     nxt.issue(min(kRecTokens, len - t0), tid, dim,
               [=](int tt, int d) { return base[(int64_t)tt * qkv_stride + (int64_t)g0 * dim + d]; },
               [=](int tt, int d) { return base[(int64_t)tt * qkv_stride + (int64_t)(G + g0) * dim + d]; },
               [=](int tt, int c) { return col0 + c < vdim ? base[(int64_t)tt * qkv_stride + (int64_t)2 * G * dim + (int64_t)h * vdim + col0 + c] : 0.f; });
+    if constexpr (CH) {
+      const int tt = tid >> 4, part = tid & 15;
+#pragma unroll
+      for (int j = 0; j < NS; ++j) {
+        const int d = part + 16 * j;
+        gnx[j] = tt < min(kRecTokens, len - t0) && d < dim ? gates[(int64_t)(row0 + t0 + tt) * gs + (int64_t)h * dim + d] : 1.f;
+      }
+    }
   };
   fetch(0);
   for (int t0 = 0; t0 < len; t0 += kRecTokens) {
@@ -151,10 +160,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     if constexpr (CH) {
       const int tt = tid >> 4, part = tid & 15;
 #pragma unroll
-      for (int j = 0; j < NS; ++j) {
-        const int d = part + 16 * j;
-        s_gc[tt][d] = tt < tc && d < dim ? gates[(int64_t)(row0 + t0 + tt) * gs + (int64_t)h * dim + d] : 1.f;
-      }
+      for (int j = 0; j < NS; ++j) s_gc[tt][part + 16 * j] = gnx[j];
     }
     __syncthreads();
     if (t0 + kRecTokens < len) fetch(t0 + kRecTokens);
