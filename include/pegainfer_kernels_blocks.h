@@ -164,6 +164,24 @@ pegainfer_status_t pegainfer_time_conv_commit(const void* in, int32_t in_dtype, 
                                               int64_t slot_stride, int32_t channels, int32_t taps, const int32_t* entry_row0,
                                               const int32_t* entry_slot, int32_t n_entries, pegainfer_stream_t stream);
 
+/* The three with biases (of w_dtype / bias_dtype, [channels], NULL = none): in_bias is part of every real input - it is added to the
+ * rows read from `in` and so also sits in the carried inputs, but not in the zeros before a sequence's start (a projection's bias
+ * ahead of the convolution); out_bias is added to the sum before the activation (the convolution's own bias). */
+pegainfer_status_t pegainfer_time_conv_biased(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w, int32_t w_dtype,
+                                              const void* in_bias, const void* out_bias, const float* state, int64_t slot_stride,
+                                              void* out, int32_t out_dtype, int64_t out_row_stride, int32_t channels, int32_t taps,
+                                              int32_t mode, const int32_t* row_entry, const int32_t* entry_row0,
+                                              const int32_t* entry_slot, int32_t n_rows, pegainfer_stream_t stream);
+pegainfer_status_t pegainfer_time_conv_step_biased(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w,
+                                                   int32_t w_dtype, const void* in_bias, const void* out_bias, float* state,
+                                                   int64_t slot_stride, void* out, int32_t out_dtype, int64_t out_row_stride,
+                                                   int32_t channels, int32_t taps, int32_t mode, const int32_t* entry_slot,
+                                                   int32_t n_entries, pegainfer_stream_t stream);
+pegainfer_status_t pegainfer_time_conv_commit_biased(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* in_bias,
+                                                     int32_t bias_dtype, float* state, int64_t slot_stride, int32_t channels,
+                                                     int32_t taps, const int32_t* entry_row0, const int32_t* entry_slot,
+                                                     int32_t n_entries, pegainfer_stream_t stream);
+
 /* RMS norm in groups on a sublayer's OUTPUT, the residual sum, and optionally a weighted sum over earlier streams:
  *   n      = y cut into `groups` equal consecutive parts, each / sqrt(mean(part^2) + eps), whole row * w
  *   r      = (x_in ? x_in : 0) + n                           -> x_out (fp32, optional), xb_out (dtype, optional)
@@ -216,6 +234,31 @@ pegainfer_status_t pegainfer_scalar_rms_add(const float* x_in, const void* y, in
                                             float eps, float* n_out, int32_t d, int32_t rows, int32_t dtype,
                                             pegainfer_stream_t stream);
 
+/* Up to three sublayer outputs join the stream in one launch, then the RMS norm (a weight per channel) of what reads the stream
+ * next.  A term with norm_w is RMS-normed over the row first:
+ *   term_t = (norm_w ? (y + bias) / sqrt(mean((y + bias)^2) + eps) * norm_w : y + bias) * factor
+ *   r = x_in + sum_t term_t                         -> x_out (fp32; may alias x_in; optional)
+ *   n = r / sqrt(mean(r^2) + eps) * gain            -> n_out (n_dtype: 1 = float, else the storage type; optional)
+ * y rows of dtype at y_row_stride; bias, norm_w, gain [d] of dtype.  x_in may be NULL when there are terms; n_terms = 0 is the
+ * plain norm of x_in. */
+typedef struct {
+  const void* y;
+  int64_t y_row_stride;
+  const void* bias;
+  const void* norm_w;
+  float factor;
+} pegainfer_sum_term;
+pegainfer_status_t pegainfer_terms_rms_add(const float* x_in, const pegainfer_sum_term* terms, int32_t n_terms, float* x_out,
+                                           const void* gain, float eps, void* n_out, int32_t n_dtype, int32_t d, int32_t rows,
+                                           int32_t dtype, pegainfer_stream_t stream);
+/* out[row, i] = act(gate[row, i]) * up[row, i], i < I; gate and up are column ranges of rows with stride in_row_stride (elements of
+ * dtype).  act 0 = silu, 1 = relu, 2 = gelu (tanh form) */
+enum { PEGAINFER_ACT_SILU = 0, PEGAINFER_ACT_RELU = 1, PEGAINFER_ACT_GELU_TANH = 2 };
+pegainfer_status_t pegainfer_glu_rows(const void* gate, const void* up, int64_t in_row_stride, void* out, int64_t out_row_stride,
+                                      int32_t I, int32_t rows, int32_t act, int32_t dtype, pegainfer_stream_t stream);
+/* out[i] = cap * tanh(in[i] / cap) over n fp32 values (in place allowed) */
+pegainfer_status_t pegainfer_softcap_rows(const float* in, float* out, int64_t n, float cap, pegainfer_stream_t stream);
+
 /* ---- recurrent matrix memories (state per (slot, head): S [dim][vdim] fp32, row-major) ----
  * Gated delta rule.  Per row, from qkv (fp32 [rows][qkv_stride]: q heads at 0, k heads at kv_heads * dim, v heads at
  * 2 * kv_heads * dim) and the projection row `proj` (dtype; beta logits at b_off, decay inputs at a_off, one per head):
@@ -250,12 +293,30 @@ pegainfer_status_t pegainfer_gated_matrix_memory(const void* proj, int64_t proj_
                                                  int32_t heads, int32_t dim, int32_t vdim, const int32_t* entry_row0,
                                                  const int32_t* entry_slot, int32_t n_entries, int32_t dtype,
                                                  pegainfer_stream_t stream);
+/* Selective state-space scan with ONE decay per head and token (state per (slot, head): S [n_state][vdim] fp32, row-major; the
+ * slot's region holds the heads back to back).  Per row from xbc (fp32 [rows][xbc_stride]: x heads * vdim at 0, B groups * n_state
+ * after it, C groups * n_state after that; head h reads group h / (heads / groups)) and the raw step size proj[row, dt_off + h]
+ * (dtype):
+ *   dt = softplus(raw + dt_bias[h]);  S <- exp(-exp(A_log[h]) dt) S + dt B x^T;  y = S^T C + D[h] x
+ * y: fp32 [rows][heads * vdim].  n_state <= 256.  Everything in fp32, the token order is fixed. */
+pegainfer_status_t pegainfer_ssd_scan(const float* xbc, int64_t xbc_stride, const void* proj, int64_t proj_stride, int64_t dt_off,
+                                      const void* A_log, const void* dt_bias, const void* D, float* state, int64_t slot_stride,
+                                      float* o, int32_t heads, int32_t groups, int32_t n_state, int32_t vdim,
+                                      const int32_t* entry_row0, const int32_t* entry_slot, int32_t n_entries, int32_t dtype,
+                                      pegainfer_stream_t stream);
 /* Per-head RMS norm of a memory's read-out, a weight, a gate and a constant factor:
  *   out[row, h, :] = o[row, h, :] / sqrt(mean(o[row, h, :]^2) + eps) * w * act(gate[row, h, :]) * factor
  * w: [vdim] shared by the heads (w_per_head == 0) or [heads * vdim]; gate_kind 0 = silu, 1 = sigmoid; gate rows of dtype
  * with stride gate_stride; out rows of dtype with stride out_stride. */
 pegainfer_status_t pegainfer_head_rms_gate(const float* o, const void* w, int32_t w_per_head, const void* gate,
                                            int64_t gate_stride, int32_t gate_kind, float factor, float eps, void* out,
+                                           int64_t out_stride, int32_t heads, int32_t vdim, int32_t rows, int32_t dtype,
+                                           pegainfer_stream_t stream);
+
+/* pegainfer_head_rms_gate with a choice of order: gate_first != 0 norms the GATED values,
+ *   out[row, h, :] = g / sqrt(mean(g^2) + eps) * w * factor,  g = o[row, h, :] * act(gate[row, h, :]) */
+pegainfer_status_t pegainfer_head_gate_rms(const float* o, const void* w, int32_t w_per_head, const void* gate, int64_t gate_stride,
+                                           int32_t gate_kind, int32_t gate_first, float factor, float eps, void* out,
                                            int64_t out_stride, int32_t heads, int32_t vdim, int32_t rows, int32_t dtype,
                                            pegainfer_stream_t stream);
 
@@ -286,6 +347,23 @@ pegainfer_status_t pegainfer_qk_prep_paged(const void* proj, int64_t proj_stride
                                           const int32_t* page_indptr, const int32_t* page_ids, void* cache, int64_t page_stride,
                                           int64_t k_cache_off, int64_t v_cache_off, int32_t page_size, float* q_out,
                                           void* q_out_stored, int32_t n_rows, int32_t dtype, pegainfer_stream_t stream);
+/* The same with a choice of where the rows come from, of the norm and of the rotation's layout.  proj_dtype: type of the rows
+ * read (the storage type, or 1 = float for rows that an fp32 stage such as a time convolution left; offsets and stride in its
+ * elements).  norm_kind HEAD_WEIGHT: per head before the rotation, times q_norm / k_norm [dim] (no norm when they are NULL);
+ * HEAD_UNIT_AFTER: per head AFTER the rotation, no weight (q_norm / k_norm unused); ALL_WEIGHT: ONE root mean square over all
+ * heads of q (of k) before the rotation, times q_norm [heads * dim] / k_norm [kv_heads * dim].  rot_layout PAIRS: neighbours
+ * (2i, 2i + 1) turn together; HALVES: value i with value i + rot_dims / 2, both by position * inv_freq[i].  dim <= 256. */
+enum { PEGAINFER_QKNORM_HEAD_WEIGHT = 0, PEGAINFER_QKNORM_HEAD_UNIT_AFTER = 1, PEGAINFER_QKNORM_ALL_WEIGHT = 2 };
+enum { PEGAINFER_ROT_PAIRS = 0, PEGAINFER_ROT_HALVES = 1 };
+pegainfer_status_t pegainfer_qk_prep_paged_form(const void* proj, int32_t proj_dtype, int64_t proj_stride, int64_t q_off,
+                                               int64_t k_off, int64_t v_off, int32_t heads, int32_t kv_heads, int32_t dim,
+                                               int32_t vdim, const void* q_norm, const void* k_norm, int32_t norm_kind, float eps,
+                                               const void* q_bias, const void* k_bias, const void* v_bias, float qt_coef,
+                                               int32_t qt_every, const float* inv_freq, int32_t rot_dims, int32_t rot_layout,
+                                               const int32_t* positions, const int32_t* row_entry, const int32_t* page_indptr,
+                                               const int32_t* page_ids, void* cache, int64_t page_stride, int64_t k_cache_off,
+                                               int64_t v_cache_off, int32_t page_size, float* q_out, void* q_out_stored,
+                                               int32_t n_rows, int32_t dtype, pegainfer_stream_t stream);
 /* Causal softmax attention, scores and weights in fp32:  out[row, h, :] = factor * sum_{j <= position} softmax_j(q . k_j * scale) v_j.
  * The rows are cut by the caller into tiles that stay inside one entry: tile i covers rows tile_row0[i] .. + tile_ntok[i] - 1
  * and, of each key/value group's query heads, tile_qh0[i] .. + tile_nqh[i] - 1, with ntok * nqh <= 16.  dim, vdim <= 256.
@@ -317,6 +395,26 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
                                                 int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
                                                 int32_t head_norm, float norm_eps, int32_t n_split, float* workspace,
                                                 int32_t plain, int32_t dtype, pegainfer_stream_t stream);
+/* The same with more ways to shape the scores.  softcap > 0: score <- softcap * tanh(score / softcap), after the scale.
+ * window > 0: a key j is visible to position i only if j <= i and (i - j < window or j < keep_first): a sliding window whose
+ * first keep_first tokens of the sequence stay visible, at their true positions; key tiles that no row of a workgroup sees are
+ * not visited.  dist_bias: fp32 [n_dist][heads] (or NULL), added to the scaled, capped score of query head h by distance,
+ * dist_bias[min(i - j, n_dist - 1)][h]: a learned bias over distance buckets, expanded by the caller to one row per distance up to
+ * the distance from which the bucket no longer changes.  gate_kind != 0: an output gate, logits of dtype in rows at gate_stride; the
+ * finished head (after norm and factor) is multiplied by sigmoid(gate[row, h * vdim + c]) (PER_VALUE) or sigmoid(gate[row, h])
+ * (PER_HEAD). */
+enum { PEGAINFER_GATE_NONE = 0, PEGAINFER_GATE_PER_VALUE = 1, PEGAINFER_GATE_PER_HEAD = 2 };
+pegainfer_status_t pegainfer_paged_attention_masked(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
+                                                    int64_t v_cache_off, int32_t page_size, const int32_t* positions,
+                                                    const int32_t* row_entry, const int32_t* page_indptr, const int32_t* page_ids,
+                                                    int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float scale,
+                                                    float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
+                                                    const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
+                                                    int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
+                                                    int32_t head_norm, float norm_eps, float softcap, int32_t window,
+                                                    int32_t keep_first, const float* dist_bias, int32_t n_dist, const void* gate,
+                                                    int64_t gate_stride, int32_t gate_kind, int32_t n_split, float* workspace,
+                                                    int32_t plain, int32_t dtype, pegainfer_stream_t stream);
 /* fp32 values of scratch a launch with n_split > 1 needs (0 for n_split <= 1) */
 int64_t pegainfer_paged_attention_workspace(int32_t n_tiles, int32_t kv_heads, int32_t vdim, int32_t maps, int32_t n_split);
 /* out[row, :cols] = in[row, :cols] * factor; rows of in / out at their own strides (elements of dtype) */

@@ -105,6 +105,8 @@ pegainfer_sched_t pegainfer_sched_create_duguzen(void* model, uint64_t seed, con
 pegainfer_sched_t pegainfer_sched_create_feruzen(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop);
 /* the same over the Ramalix runtime (pegainfer_ramalix.h): `model` is a pegainfer_ramalix_t */
 pegainfer_sched_t pegainfer_sched_create_ramalix(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop);
+/* the same over the Kukulorn runtime (pegainfer_kukulorn.h): `model` is a pegainfer_kukulorn_t */
+pegainfer_sched_t pegainfer_sched_create_kukulorn(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop);
 void pegainfer_sched_destroy(pegainfer_sched_t s);
 
 /* EngineHandle::submit: returns the RequestId the events carry (ids count up from 0 in submission order) */

@@ -1,6 +1,6 @@
 // Softmax attention over a paged key/value cache for any head sizes and grouped key/value heads, in a bf16 and an fp32
 // storage instance; norms, angles, scores, softmax state and accumulators are fp32 in both.
-//   qk_norm_rope_paged_kernel  one workgroup per token row, a wave per head: optional bias, optional RMS norm over the head
+//   qk_prep_paged_kernel       one workgroup per token row, a wave per head: optional bias, optional RMS norm over the head
 //                              (plain weight), optional position-dependent query factor (query temperature), rotation
 //                              of neighbouring pairs (2i, 2i + 1) of the first rot_dims values by position * inv_freq[i],
 //                              queries to an fp32 buffer, keys and values into the cache entry of (request, position)
@@ -22,61 +22,112 @@
 
 namespace pk {
 
-template <typename A>
-__global__ __launch_bounds__(256) void qk_norm_rope_paged_kernel(
-    const A* __restrict__ proj, int64_t proj_stride, int64_t q_off, int64_t k_off, int64_t v_off, int H, int G, int dim, int vdim,
+// how qk_prep_paged_kernel norms and rotates
+struct PrepForm {
+  int norm_kind = 0;    // 0: per head before the rotation, times a weight [dim] (when weights are given); 1: per head AFTER the
+                        // rotation, no weight (unit root mean square); 2: over ALL heads of the projection at once before the
+                        // rotation, times a weight [heads * dim] / [kv_heads * dim]
+  int rot_halves = 0;   // 0: neighbours (2i, 2i + 1) are rotated together; 1: value i with value i + rot_dims / 2
+};
+
+// I: type of the projection rows read (the storage type, or float for rows that an fp32 stage such as a convolution left)
+template <typename A, typename I>
+__global__ __launch_bounds__(256) void qk_prep_paged_kernel(
+    const I* __restrict__ proj, int64_t proj_stride, int64_t q_off, int64_t k_off, int64_t v_off, int H, int G, int dim, int vdim,
     const A* __restrict__ q_norm, const A* __restrict__ k_norm, float eps, const float* __restrict__ inv_freq, int rot_dims,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_entry, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ page_ids, A* __restrict__ cache, int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
     int page_size, float* __restrict__ q_out, A* __restrict__ q_out_stored, const A* __restrict__ q_bias,
-    const A* __restrict__ k_bias, const A* __restrict__ v_bias, float qt_coef, int qt_every) {
+    const A* __restrict__ k_bias, const A* __restrict__ v_bias, float qt_coef, int qt_every, PrepForm pf) {
   extern __shared__ float sm[];   // [4 waves][dim]
+  __shared__ float red[4];
   const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pos = positions[row], e = row_entry[row];
   const int64_t page = page_ids[page_indptr[e] + pos / page_size];
   const int slot = pos % page_size;
-  const A* pr = proj + (int64_t)row * proj_stride;
+  const I* pr = proj + (int64_t)row * proj_stride;
   float* buf = sm + wave * dim;
   // query temperature: a factor on the whole query that grows with the logarithm of the position's block number
   const float qt = qt_every > 0 ? 1.0f + qt_coef * logf((float)((pos + 1) / qt_every) + 1.0f) : 1.0f;
+  float inv_all_q = 1.f, inv_all_k = 1.f;
+  if (pf.norm_kind == 2) {   // root mean squares over the whole q and the whole k projection
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < H * dim; i += 256) {
+      const float v = ld(pr + q_off + i) + (q_bias ? ld(q_bias + i) : 0.f);
+      sq = fmaf(v, v, sq);
+    }
+    for (int i = threadIdx.x; i < G * dim; i += 256) {
+      const float v = ld(pr + k_off + i) + (k_bias ? ld(k_bias + i) : 0.f);
+      sk = fmaf(v, v, sk);
+    }
+    inv_all_q = 1.0f / sqrtf(block_sum<4>(sq, red) / (float)(H * dim) + eps);
+    inv_all_k = 1.0f / sqrtf(block_sum<4>(sk, red) / (float)(G * dim) + eps);
+  }
+  const int half = rot_dims >> 1;
   for (int hh = wave; hh < H + G; hh += 4) {
     const bool is_q = hh < H;
-    const A* src = is_q ? pr + q_off + (int64_t)hh * dim : pr + k_off + (int64_t)(hh - H) * dim;
+    const int hd = is_q ? hh : hh - H;
+    const I* src = is_q ? pr + q_off + (int64_t)hd * dim : pr + k_off + (int64_t)hd * dim;
     const A* nw = is_q ? q_norm : k_norm;
-    const A* bs = is_q ? (q_bias ? q_bias + (int64_t)hh * dim : nullptr) : (k_bias ? k_bias + (int64_t)(hh - H) * dim : nullptr);
+    const A* bs = is_q ? (q_bias ? q_bias + (int64_t)hd * dim : nullptr) : (k_bias ? k_bias + (int64_t)hd * dim : nullptr);
     float ss = 0.f;
     for (int i = lane; i < dim; i += 64) {
       const float v = ld(src + i) + (bs ? ld(bs + i) : 0.f);
       buf[i] = v;
       ss = fmaf(v, v, ss);
     }
-    if (nw) {
+    if (pf.norm_kind == 0 && nw) {
       ss = wave_sum(ss);
       const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
       for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * ld(nw + i);
+    } else if (pf.norm_kind == 2) {
+      const float inv = is_q ? inv_all_q : inv_all_k;
+      for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * ld(nw + (int64_t)hd * dim + i);
     }
     if (is_q && qt_every > 0)
       for (int i = lane; i < dim; i += 64) buf[i] *= qt;
     __builtin_amdgcn_wave_barrier();
-    for (int i = lane; i < dim; i += 64) {
-      float out = buf[i];
-      if (i < rot_dims) {
-        const float ang = (float)pos * inv_freq[i >> 1];
-        const float c = cosf(ang), s = sinf(ang);
-        out = (i & 1) ? buf[i] * c + buf[i - 1] * s : buf[i] * c - buf[i + 1] * s;
+    float keep[4];   // dim <= 256: a lane's values i = lane, lane + 64, ...
+    float ss2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int i = lane + 64 * c;
+      float out = 0.f;
+      if (i < dim) {
+        out = buf[i];
+        if (i < rot_dims) {
+          if (pf.rot_halves) {
+            const int f = i < half ? i : i - half;
+            const float ang = (float)pos * inv_freq[f];
+            const float cs = cosf(ang), sn = sinf(ang);
+            out = i < half ? buf[i] * cs - buf[i + half] * sn : buf[i] * cs + buf[i - half] * sn;
+          } else {
+            const float ang = (float)pos * inv_freq[i >> 1];
+            const float cs = cosf(ang), sn = sinf(ang);
+            out = (i & 1) ? buf[i] * cs + buf[i - 1] * sn : buf[i] * cs - buf[i + 1] * sn;
+          }
+        }
+        ss2 = fmaf(out, out, ss2);
       }
+      keep[c] = out;
+    }
+    const float post = pf.norm_kind == 1 ? 1.0f / sqrtf(wave_sum(ss2) / (float)dim + eps) : 1.0f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int i = lane + 64 * c;
+      if (i >= dim) continue;
+      const float out = keep[c] * post;
       if (is_q) {
         if (q_out_stored) st(q_out_stored + ((int64_t)row * H + hh) * dim + i, out);
         else q_out[((int64_t)row * H + hh) * dim + i] = out;
       } else
-        st(cache + page * page_stride + k_cache_off + ((int64_t)slot * G + (hh - H)) * dim + i, out);
+        st(cache + page * page_stride + k_cache_off + ((int64_t)slot * G + hd) * dim + i, out);
     }
     __builtin_amdgcn_wave_barrier();
   }
   for (int i = threadIdx.x; i < G * vdim; i += 256) {
     A* dst = cache + page * page_stride + v_cache_off + (int64_t)slot * G * vdim + i;
-    if (v_bias) st(dst, ld(pr + v_off + i) + ld(v_bias + i));
-    else *dst = pr[v_off + i];
+    st(dst, ld(pr + v_off + i) + (v_bias ? ld(v_bias + i) : 0.f));
   }
 }
 
@@ -93,13 +144,35 @@ struct AttnForm {
                                // key head holds [map 1 : dim | map 2 : dim])
   int head_norm = 0;           // != 0: out / sqrt(mean(out^2) + norm_eps) over the head's vdim values, before `factor`
   float norm_eps = 0.f;
+  float softcap = 0.f;         // > 0: score <- softcap * tanh(score / softcap), after the scale
+  int window = 0;              // > 0: a key j is visible to position i only if i - j < window or j < keep_first (kept first
+  int keep_first = 0;          // tokens stay visible at their true positions)
+  const float* dist_bias = nullptr;   // fp32 [n_dist][heads], added to the (scaled, capped) score of query head h by distance:
+  int n_dist = 0;                     // dist_bias[min(i - j, n_dist - 1)][h]
+  const void* gate = nullptr;  // output gate logits (storage type), rows at gate_stride: the finished head is multiplied by
+  int64_t gate_stride = 0;     // sigmoid(gate[row, h * vdim + c]) (gate_kind 1: one per value) or sigmoid(gate[row, h]) (2: one
+  int gate_kind = 0;           // per head)
 };
+
+// first position of the run of keys that position `pos` sees (besides the kept first tokens)
+__device__ __forceinline__ int attn_row_lo(const AttnForm& form, int pos) {
+  int lo = form.block > 0 ? (pos / form.block) * form.block : 0;
+  if (form.window > 0) lo = max(lo, pos - form.window + 1);
+  return lo;
+}
+// a raw dot product turned into the score of (query position rpos, key position kp, query head qh)
+__device__ __forceinline__ float attn_score(const AttnForm& form, float dot, float scale, int rpos, int kp, int qh, int H) {
+  float sc = dot * scale;
+  if (form.softcap > 0.f) sc = form.softcap * tanhf(sc / form.softcap);
+  if (form.dist_bias) sc += form.dist_bias[(int64_t)min(rpos - kp, form.n_dist - 1) * H + qh];
+  return sc;
+}
 
 // A row's softmax states (one per map) turned into its output: the sink joins every denominator, the maps are combined, the
 // head is normed, `factor` comes last.  The wave holds the row: lane l has columns l, l + 64, ...
 template <typename A, int MAPS>
-__device__ __forceinline__ void attn_finish_row(float* mrun, float* lrun, float (*acc)[4], const AttnForm& form, int qh, int vdim,
-                                                float factor, int lane, A* __restrict__ dst) {
+__device__ __forceinline__ void attn_finish_row(float* mrun, float* lrun, float (*acc)[4], const AttnForm& form, int row, int qh,
+                                                int vdim, float factor, int lane, A* __restrict__ dst) {
   float res[4];
   if (form.sink) {   // rescale to the larger of the two maxima first
     const float sk = ld(static_cast<const A*>(form.sink) + qh);
@@ -129,9 +202,15 @@ __device__ __forceinline__ void attn_finish_row(float* mrun, float* lrun, float 
       if (lane + 64 * c < vdim) ss = fmaf(res[c], res[c], ss);
     post = factor / sqrtf(wave_sum(ss) / (float)vdim + form.norm_eps);
   }
+  if (form.gate_kind == 2) post *= sigmoid_f(ld(static_cast<const A*>(form.gate) + (int64_t)row * form.gate_stride + qh));
 #pragma unroll
   for (int c = 0; c < 4; ++c)
-    if (lane + 64 * c < vdim) st(dst + lane + 64 * c, res[c] * post);
+    if (lane + 64 * c < vdim) {
+      float v = res[c] * post;
+      if (form.gate_kind == 1)
+        v *= sigmoid_f(ld(static_cast<const A*>(form.gate) + (int64_t)row * form.gate_stride + (int64_t)qh * vdim + lane + 64 * c));
+      st(dst + lane + 64 * c, v);
+    }
 }
 
 template <typename A, int MAPS>
@@ -160,19 +239,21 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   const int32_t* pages = page_ids + page_indptr[e];
   const int kmax = positions[row0 + ntok - 1] + 1;    // keys 0 .. kmax - 1 are visible to the tile's last token
   // the first key any row of the tile sees, rounded down to the 64-key grid that starts at position 0
-  const int kfirst = form.block > 0 ? ((positions[row0] / form.block) * form.block / kAttKeys) * kAttKeys : 0;
+  const int lo0 = attn_row_lo(form, positions[row0]);   // rows of a tile are in position order: the lowest run start
+  const int kfirst = form.keep_first > 0 ? 0 : (lo0 / kAttKeys) * kAttKeys;
   for (int i = tid; i < nrows * qd; i += 256) {
     const int lr = i / qd, d = i % qd;
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
     s_q[lr * qd + d] = q[((int64_t)(row0 + tok) * H + qh) * qd + d];
   }
   float mrun[kAttRpw][MAPS], lrun[kAttRpw][MAPS], acc[kAttRpw][MAPS][4];
-  int rpos[kAttRpw], rlo[kAttRpw];
+  int rpos[kAttRpw], rlo[kAttRpw], rqh[kAttRpw];
 #pragma unroll
   for (int i = 0; i < kAttRpw; ++i) {
     const int lr = wave + 4 * i;
     rpos[i] = lr < nrows ? positions[row0 + lr / nqh] : -1;
-    rlo[i] = form.block > 0 && rpos[i] >= 0 ? (rpos[i] / form.block) * form.block : 0;
+    rlo[i] = rpos[i] >= 0 ? attn_row_lo(form, rpos[i]) : 0;
+    rqh[i] = g * per_group + qh0 + (lr < nrows ? lr % nqh : 0);
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
       mrun[i][m] = -INFINITY;
@@ -185,6 +266,8 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   // context's length, so a recorded launch serves every later length) and leaves its softmax state to the merge kernel
   for (int k0 = kfirst + (int)blockIdx.z * kAttKeys; k0 < kmax; k0 += kAttKeys * nsplit) {
     const int nk = min(kAttKeys, kmax - k0);
+    // a tile between the kept first tokens and the lowest run start is seen by no row (uniform over the workgroup)
+    if (k0 >= form.keep_first && k0 + kAttKeys <= lo0) continue;
     __syncthreads();
     {   // staging: four threads per key; one page lookup per thread and tile, 16-byte loads where the layout allows
       const int j = tid >> 2, sub = tid & 3;
@@ -226,10 +309,10 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
     for (int i = 0; i < kAttRpw; ++i) {
       const int lr = wave + 4 * i;
       // a row whose position lies before the tile, or whose run of visible keys begins after it, is left as it is
-      act[i] = lr < nrows && k0 <= rpos[i] && k0 + nk > rlo[i];
+      act[i] = lr < nrows && k0 <= rpos[i] && (k0 + nk > rlo[i] || k0 < form.keep_first);
       if (act[i]) {
         any = true;
-        jlo = min(jlo, max(0, rlo[i] - k0));
+        jlo = min(jlo, k0 < form.keep_first ? 0 : max(0, rlo[i] - k0));
         jhi = max(jhi, min(nk, rpos[i] - k0 + 1));
       }
     }
@@ -267,8 +350,9 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
         corr[i] = 1.0f;
         float pv = 0.f;
         if (act[i]) {
-          const bool seen = lane < nk && k0 + lane <= rpos[i] && k0 + lane >= rlo[i];
-          const float sc = seen ? a[i] * scale : -INFINITY;
+          const int kp_ = k0 + lane;
+          const bool seen = lane < nk && kp_ <= rpos[i] && (kp_ >= rlo[i] || kp_ < form.keep_first);
+          const float sc = seen ? attn_score(form, a[i], scale, rpos[i], kp_, rqh[i], H) : -INFINITY;
           const float mnew = fmaxf(mrun[i][m], wave_max(sc));
           pv = sc == -INFINITY ? 0.f : expf(sc - mnew);
           corr[i] = mrun[i][m] == -INFINITY ? 0.f : expf(mrun[i][m] - mnew);
@@ -320,7 +404,7 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
     const int lr = wave + 4 * i;
     if (lr >= nrows) continue;
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
-    attn_finish_row<A, MAPS>(mrun[i], lrun[i], acc[i], form, qh, vdim, factor, lane,
+    attn_finish_row<A, MAPS>(mrun[i], lrun[i], acc[i], form, row0 + tok, qh, vdim, factor, lane,
                              out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
   }
 }
@@ -361,7 +445,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int e = row_entry[row0];
   const int32_t* pages = page_ids + page_indptr[e];
   const int kmax = positions[row0 + ntok - 1] + 1;
-  const int kfirst = form.block > 0 ? ((positions[row0] / form.block) * form.block / kAttKeys) * kAttKeys : 0;
+  const int lo0 = attn_row_lo(form, positions[row0]);   // rows of a tile are in position order: the lowest run start
+  const int kfirst = form.keep_first > 0 ? 0 : (lo0 / kAttKeys) * kAttKeys;
   // zeros everywhere first: padding columns, rows past the tile's, keys past the context's end must multiply as zeros
   for (int i = tid; i < (kAttKeys + kAttRows) * ks + VP * kMfVs; i += 256) s_k[i] = 0;
   __syncthreads();
@@ -371,7 +456,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     s_q[lr * ks + (c / dim) * dp + c % dim] = f2bf(q[((int64_t)(row0 + tok) * H + qh) * qd + c]);
   }
   const int rpos = lrow < nrows ? positions[row0 + lrow / nqh] : -1;      // this lane's row (as a column of S^T)
-  const int rlo = form.block > 0 && rpos >= 0 ? (rpos / form.block) * form.block : 0;
+  const int rlo = rpos >= 0 ? attn_row_lo(form, rpos) : 0;
+  const int lqh = g * per_group + qh0 + (lrow < nrows ? lrow % nqh : 0);
   float mrun[MAPS], lrun[MAPS];
   f32x4 o[MAPS][NCB];
 #pragma unroll
@@ -385,6 +471,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const bool vec_v = (vdim & 7) == 0 && (page_stride & 7) == 0 && (v_cache_off & 7) == 0 && aligned16(cache);
   for (int k0 = kfirst + (int)blockIdx.z * kAttKeys; k0 < kmax; k0 += kAttKeys * nsplit) {
     const int nk = min(kAttKeys, kmax - k0);
+    if (k0 >= form.keep_first && k0 + kAttKeys <= lo0) continue;   // seen by no row of the tile (uniform over the workgroup)
     __syncthreads();
     {   // staging: four threads per key; the value tile is written transposed
       const int j = tid >> 2, sub = tid & 3;
@@ -435,7 +522,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int kp_ = k0 + kb + 4 * lgrp + r;
-        sv[r] = (kp_ <= rpos && kp_ >= rlo) ? sv[r] * scale : -INFINITY;
+        sv[r] = (kp_ <= rpos && (kp_ >= rlo || kp_ < form.keep_first)) ? attn_score(form, sv[r], scale, rpos, kp_, lqh, H) : -INFINITY;
         tmax = fmaxf(tmax, sv[r]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
@@ -544,7 +631,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       continue;
     }
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
-    attn_finish_row<uint16_t, MAPS>(fm, fl, acc, form, qh, vdim, factor, lane, out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
+    attn_finish_row<uint16_t, MAPS>(fm, fl, acc, form, row0 + tok, qh, vdim, factor, lane, out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
   }
 }
 
@@ -598,7 +685,7 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(
       }
     }
     const int tok = lr / nqh, qh = g * per_group + qh0 + lr % nqh;
-    attn_finish_row<A, MAPS>(mrun, lrun, acc, form, qh, vdim, factor, lane, out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
+    attn_finish_row<A, MAPS>(mrun, lrun, acc, form, row0 + tok, qh, vdim, factor, lane, out + (int64_t)(row0 + tok) * out_stride + (int64_t)qh * vdim);
   }
 }
 
@@ -626,21 +713,42 @@ pegainfer_status_t pegainfer_qk_prep_paged(const void* proj, int64_t proj_stride
                                           const int32_t* page_indptr, const int32_t* page_ids, void* cache, int64_t page_stride,
                                           int64_t k_cache_off, int64_t v_cache_off, int32_t page_size, float* q_out,
                                           void* q_out_stored, int32_t n_rows, int32_t dtype, pegainfer_stream_t stream) {
+  return pegainfer_qk_prep_paged_form(proj, dtype, proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim, q_norm, k_norm,
+                                      PEGAINFER_QKNORM_HEAD_WEIGHT, eps, q_bias, k_bias, v_bias, qt_coef, qt_every, inv_freq, rot_dims,
+                                      PEGAINFER_ROT_PAIRS, positions, row_entry, page_indptr, page_ids, cache, page_stride, k_cache_off,
+                                      v_cache_off, page_size, q_out, q_out_stored, n_rows, dtype, stream);
+}
+
+pegainfer_status_t pegainfer_qk_prep_paged_form(const void* proj, int32_t proj_dtype, int64_t proj_stride, int64_t q_off,
+                                               int64_t k_off, int64_t v_off, int32_t heads, int32_t kv_heads, int32_t dim,
+                                               int32_t vdim, const void* q_norm, const void* k_norm, int32_t norm_kind, float eps,
+                                               const void* q_bias, const void* k_bias, const void* v_bias, float qt_coef,
+                                               int32_t qt_every, const float* inv_freq, int32_t rot_dims, int32_t rot_layout,
+                                               const int32_t* positions, const int32_t* row_entry, const int32_t* page_indptr,
+                                               const int32_t* page_ids, void* cache, int64_t page_stride, int64_t k_cache_off,
+                                               int64_t v_cache_off, int32_t page_size, float* q_out, void* q_out_stored,
+                                               int32_t n_rows, int32_t dtype, pegainfer_stream_t stream) {
   if (n_rows <= 0) return 0;
-  if (heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims > dim || (rot_dims & 1) || page_size <= 0 ||
-      (rot_dims > 0 && !inv_freq) || (!q_norm) != (!k_norm) || (size_t)4 * dim * sizeof(float) > 64 * 1024)
+  if (heads <= 0 || kv_heads <= 0 || dim <= 0 || dim > 256 || vdim <= 0 || rot_dims < 0 || rot_dims > dim || (rot_dims & 1) ||
+      page_size <= 0 || (rot_dims > 0 && !inv_freq) || (!q_norm) != (!k_norm) || norm_kind < 0 || norm_kind > 2 ||
+      (norm_kind == PEGAINFER_QKNORM_ALL_WEIGHT && !q_norm) || (rot_layout != PEGAINFER_ROT_PAIRS && rot_layout != PEGAINFER_ROT_HALVES))
     return PK_BAD;
-  if (!by_dtype(dtype, [&](auto* t) {
-        using A = std::remove_pointer_t<decltype(t)>;
-        qk_norm_rope_paged_kernel<A><<<n_rows, 256, (size_t)4 * dim * sizeof(float), as_stream(stream)>>>(
-            static_cast<const A*>(proj), proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim,
-            static_cast<const A*>(q_norm), static_cast<const A*>(k_norm), eps, inv_freq, rot_dims, positions, row_entry,
-            page_indptr, page_ids, static_cast<A*>(cache), page_stride, k_cache_off, v_cache_off, page_size, q_out,
-            static_cast<A*>(q_out_stored), static_cast<const A*>(q_bias), static_cast<const A*>(k_bias),
-            static_cast<const A*>(v_bias), qt_coef, qt_every);
-      }))
-    return PK_BAD;
-  return (pegainfer_status_t)hipGetLastError();
+  PrepForm pf;
+  pf.norm_kind = norm_kind;
+  pf.rot_halves = rot_layout == PEGAINFER_ROT_HALVES;
+  bool ok = true;
+  const bool known = by_dtype(dtype, [&](auto* t) {
+    using A = std::remove_pointer_t<decltype(t)>;
+    ok = by_dtype(proj_dtype, [&](auto* ti) {
+      using I = std::remove_pointer_t<decltype(ti)>;
+      qk_prep_paged_kernel<A, I><<<n_rows, 256, (size_t)4 * dim * sizeof(float), as_stream(stream)>>>(
+          static_cast<const I*>(proj), proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim, static_cast<const A*>(q_norm),
+          static_cast<const A*>(k_norm), eps, inv_freq, rot_dims, positions, row_entry, page_indptr, page_ids, static_cast<A*>(cache),
+          page_stride, k_cache_off, v_cache_off, page_size, q_out, static_cast<A*>(q_out_stored), static_cast<const A*>(q_bias),
+          static_cast<const A*>(k_bias), static_cast<const A*>(v_bias), qt_coef, qt_every, pf);
+    });
+  });
+  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
 }
 
 pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_stride, int64_t q_off, int64_t k_off,
@@ -666,7 +774,26 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
                                                 int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
                                                 int32_t head_norm, float norm_eps, int32_t n_split, float* workspace,
                                                 int32_t plain, int32_t dtype, pegainfer_stream_t stream) {
+  return pegainfer_paged_attention_masked(q, cache, page_stride, k_cache_off, v_cache_off, page_size, positions, row_entry, page_indptr,
+                                          page_ids, heads, kv_heads, dim, vdim, scale, factor, tile_row0, tile_ntok, tile_qh0, tile_nqh,
+                                          n_tiles, out, out_stride, maps, lambda, block, sink, head_norm, norm_eps, 0.f, 0, 0, nullptr, 0,
+                                          nullptr, 0, 0, n_split, workspace, plain, dtype, stream);
+}
+
+pegainfer_status_t pegainfer_paged_attention_masked(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
+                                                    int64_t v_cache_off, int32_t page_size, const int32_t* positions,
+                                                    const int32_t* row_entry, const int32_t* page_indptr, const int32_t* page_ids,
+                                                    int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float scale,
+                                                    float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
+                                                    const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
+                                                    int64_t out_stride, int32_t maps, float lambda, int32_t block, const void* sink,
+                                                    int32_t head_norm, float norm_eps, float softcap, int32_t window,
+                                                    int32_t keep_first, const float* dist_bias, int32_t n_dist, const void* gate,
+                                                    int64_t gate_stride, int32_t gate_kind, int32_t n_split, float* workspace,
+                                                    int32_t plain, int32_t dtype, pegainfer_stream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (gate_kind < 0 || gate_kind > 2 || (gate_kind && !gate)) return PK_BAD;
+  if (window < 0 || keep_first < 0 || (keep_first > 0 && window <= 0) || softcap < 0.f || (dist_bias && n_dist < 1)) return PK_BAD;
   if (n_split < 1) n_split = 1;
   if (n_split > 1 && (!workspace || n_split > 64)) return PK_BAD;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || (maps != 1 && maps != 2) || maps * dim > 256 || vdim <= 0 ||
@@ -681,6 +808,14 @@ pegainfer_status_t pegainfer_paged_attention_ex(const float* q, const void* cach
   form.lambda = lambda;
   form.head_norm = head_norm;
   form.norm_eps = norm_eps;
+  form.softcap = softcap;
+  form.window = window;
+  form.keep_first = window > 0 ? keep_first : 0;
+  form.dist_bias = dist_bias;
+  form.n_dist = n_dist;
+  form.gate = gate;
+  form.gate_stride = gate_stride;
+  form.gate_kind = gate_kind;
   bool ok = true;
   if (dtype == kDtBf16 && !plain) {   // bf16 cache: the matrix-core kernel; same tiles, same splits, same merge
     const int ncb = vdim <= 32 ? 2 : vdim <= 64 ? 4 : vdim <= 128 ? 8 : 16;

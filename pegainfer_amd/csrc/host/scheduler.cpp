@@ -14,6 +14,7 @@
 #include "pegainfer_duguzen.h"
 #include "pegainfer_feruzen.h"
 #include "pegainfer_ramalix.h"
+#include "pegainfer_kukulorn.h"
 #include "pegainfer_scheduler.h"
 
 namespace psched {
@@ -277,7 +278,7 @@ struct Qwen35Exec {
   }
 };
 
-// Executor over a runtime with ONE batched step function (pegainfer_duguzen.h, pegainfer_feruzen.h, pegainfer_ramalix.h).  The step takes prompts
+// Executor over a runtime with ONE batched step function (pegainfer_duguzen.h, pegainfer_feruzen.h, pegainfer_ramalix.h, pegainfer_kukulorn.h).  The step takes prompts
 // and single tokens of several requests as ONE batch, so a Prefill, a Decode and a Unified plan are all the same call;
 // sampled requests draw from their wanted row afterwards, logprobs read the row's fp32 logits.  Api names the runtime's
 // entry points.
@@ -303,6 +304,7 @@ struct Qwen35Exec {
 PEGAINFER_STEP_API(DuguzenApi, pegainfer_duguzen);
 PEGAINFER_STEP_API(FeruzenApi, pegainfer_feruzen);
 PEGAINFER_STEP_API(RamalixApi, pegainfer_ramalix);
+PEGAINFER_STEP_API(KukulornApi, pegainfer_kukulorn);
 
 template <class Api>
 struct StepExec {
@@ -368,6 +370,7 @@ struct StepExec {
 using DuguzenExec = StepExec<DuguzenApi>;
 using FeruzenExec = StepExec<FeruzenApi>;
 using RamalixExec = StepExec<RamalixApi>;
+using KukulornExec = StepExec<KukulornApi>;
 
 struct Scheduler {
   pegainfer_executor_vtbl ex;
@@ -376,6 +379,7 @@ struct Scheduler {
   DuguzenExec* owned_dz = nullptr;
   FeruzenExec* owned_fz = nullptr;
   RamalixExec* owned_rx = nullptr;
+  KukulornExec* owned_kk = nullptr;
   Rng rng;
   std::vector<Active> active;
   std::vector<Pending> deferred;
@@ -671,6 +675,19 @@ pegainfer_sched_t pegainfer_sched_create_ramalix(void* model, uint64_t seed, con
   s->owned_rx = e;
   return s;
 }
+pegainfer_sched_t pegainfer_sched_create_kukulorn(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop) {
+  if (!model) return nullptr;
+  auto* e = new psched::KukulornExec();
+  e->model = model;
+  for (int i = 0; i < n_stop; ++i) e->stop.insert(stop_tokens[i]);
+  pegainfer_executor_vtbl v{sizeof(pegainfer_executor_vtbl), e, &psched::KukulornExec::page_size, &psched::KukulornExec::max_request_pages,
+                            &psched::KukulornExec::available_pages, &psched::KukulornExec::is_stop_token,
+                            &psched::KukulornExec::drop_request, &psched::KukulornExec::execute, &psched::KukulornExec::last_error,
+                            &psched::KukulornExec::max_batch_size, &psched::KukulornExec::logprobs, nullptr, nullptr};
+  Scheduler* s = static_cast<Scheduler*>(pegainfer_sched_create(&v, seed));
+  s->owned_kk = e;
+  return s;
+}
 void pegainfer_sched_destroy(pegainfer_sched_t s) {
   if (!s) return;
   delete SC(s)->owned;
@@ -678,6 +695,7 @@ void pegainfer_sched_destroy(pegainfer_sched_t s) {
   delete SC(s)->owned_dz;
   delete SC(s)->owned_fz;
   delete SC(s)->owned_rx;
+  delete SC(s)->owned_kk;
   delete SC(s);
 }
 uint64_t pegainfer_sched_submit_ex(pegainfer_sched_t s, const uint32_t* prompt_tokens, int32_t n_tokens, int32_t max_tokens,

@@ -12,6 +12,7 @@
 // A round's sixteen outputs of a column leave in one store per lane.
 //   delta_rule_kernel      S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //   matrix_memory_kernel   m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;  n likewise;  o = S^T q / (max(|n.q|, e^-m') + 1e-6)
+//   ssd_scan_kernel        a = exp(-exp(A_log) dt);  S <- a S + dt B x^T;  y = S^T C + D x          (dt = softplus(raw + bias))
 // A row's result depends only on the rows before it in its own request: the token order is fixed, and cutting a prompt into
 // steps only moves where the state passes through HBM (exactly, it is fp32 either way).
 #include "common.h"
@@ -300,6 +301,82 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(const A* __restrict_
   if (blockIdx.x == 0 && tid == 0) *m_g = s_m[0];
 }
 
+// Selective state-space scan with a scalar decay per head (the state-space-duality form).  State per (slot, head): S [N][vdim].
+// xbc: fp32 rows [x: heads * vdim | B: groups * N | C: groups * N] (after their convolution and activation); the raw step sizes
+// come from the projection row (storage type), one per head.  B plays the key's part, C the query's, x the value's; no sum of a
+// token feeds the state, so four tokens' read-outs are in flight together.
+template <int NS, typename A>
+__global__ __launch_bounds__(256) void ssd_scan_kernel(const float* __restrict__ xbc, int64_t xbc_stride, const A* __restrict__ proj,
+                                                       int64_t proj_stride, int64_t dt_off, const A* __restrict__ A_log,
+                                                       const A* __restrict__ dt_bias, const A* __restrict__ Dskip,
+                                                       float* __restrict__ state, int64_t slot_stride, float* __restrict__ o, int H,
+                                                       int G, int dim, int vdim, const int32_t* __restrict__ entry_row0,
+                                                       const int32_t* __restrict__ entry_slot) {
+  constexpr int DP = kRecSlices * NS;
+  __shared__ __attribute__((aligned(16))) float s_k[kRecTokens][DP], s_q[kRecTokens][DP];
+  __shared__ float s_v[kRecTokens][kRecCols], s_a[kRecTokens], s_b[kRecTokens];
+  const int e = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kRecCols;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, cl = wave * 4 + (lane >> 4);
+  const int col = col0 + cl;
+  const int g0 = h / (H / G);
+  const int row0 = entry_row0[e], len = entry_row0[e + 1] - row0;
+  float* S_g = state + (int64_t)entry_slot[e] * slot_stride + (int64_t)h * dim * vdim;
+  float S[NS];
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    const int d = r * NS + i;
+    S[i] = d < dim && col < vdim ? S_g[(int64_t)d * vdim + col] : 0.f;
+  }
+  const float rate = -expf(ld(A_log + h)), dtb = ld(dt_bias + h), skip = ld(Dskip + h);
+  const int64_t b_at = (int64_t)H * vdim + (int64_t)g0 * dim, c_at = (int64_t)H * vdim + (int64_t)(G + g0) * dim;
+  RoundFetch<NS> nxt;
+  auto fetch = [&](int t0) {
+    const float* base = xbc + (int64_t)(row0 + t0) * xbc_stride;
+    nxt.issue(min(kRecTokens, len - t0), tid, dim,
+              [=](int tt, int d) { return base[(int64_t)tt * xbc_stride + c_at + d]; },
+              [=](int tt, int d) { return base[(int64_t)tt * xbc_stride + b_at + d]; },
+              [=](int tt, int c) { return col0 + c < vdim ? base[(int64_t)tt * xbc_stride + (int64_t)h * vdim + col0 + c] : 0.f; });
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < len; t0 += kRecTokens) {
+    const int tc = min(kRecTokens, len - t0);
+    __syncthreads();
+    nxt.land(tid, s_q, s_k, s_v);
+    if (tid < kRecTokens) {   // rows past the entry's end: a = 1, b = 0 - a step that leaves S as it is
+      const bool live = tid < tc;
+      const float dt = live ? softplus_f(ld(proj + (int64_t)(row0 + t0 + tid) * proj_stride + dt_off + h) + dtb) : 0.f;
+      s_a[tid] = live ? expf(rate * dt) : 1.f;
+      s_b[tid] = dt;
+    }
+    __syncthreads();
+    if (t0 + kRecTokens < len) fetch(t0 + kRecTokens);
+    float okeep = 0.f;
+    for (int t4 = 0; t4 < tc; t4 += 4) {
+#pragma unroll
+     for (int uu = 0; uu < 4; ++uu) {
+      const int tt = t4 + uu;
+      const float a = s_a[tt], xv = s_v[tt][cl];
+      const float bv = s_b[tt] * xv;
+      float y0 = 0.f, y1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        const float kk = s_k[tt][r * NS + i], qq = s_q[tt][r * NS + i];
+        S[i] = fmaf(bv, kk, a * S[i]);
+        if (i & 1) y1 = fmaf(S[i], qq, y1); else y0 = fmaf(S[i], qq, y0);
+      }
+      const float y = fmaf(skip, xv, row16_sum(y0 + y1));
+      okeep = tt == r ? y : okeep;
+     }
+    }
+    if (r < tc && col < vdim) o[(int64_t)(row0 + t0 + r) * ((int64_t)H * vdim) + (int64_t)h * vdim + col] = okeep;
+  }
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    const int d = r * NS + i;
+    if (d < dim && col < vdim) S_g[(int64_t)d * vdim + col] = S[i];
+  }
+}
+
 template <typename F>
 inline bool by_slices(int dim, F&& fn) {
   if (dim <= 16) fn(std::integral_constant<int, 1>());
@@ -391,3 +468,26 @@ pegainfer_status_t pegainfer_gated_matrix_memory(const void* proj, int64_t proj_
 }
 
 }  // extern "C"
+
+extern "C" pegainfer_status_t pegainfer_ssd_scan(const float* xbc, int64_t xbc_stride, const void* proj, int64_t proj_stride,
+                                                 int64_t dt_off, const void* A_log, const void* dt_bias, const void* D, float* state,
+                                                 int64_t slot_stride, float* o, int32_t heads, int32_t groups, int32_t n_state,
+                                                 int32_t vdim, const int32_t* entry_row0, const int32_t* entry_slot,
+                                                 int32_t n_entries, int32_t dtype, pegainfer_stream_t stream) {
+  using namespace pk;
+  if (n_entries <= 0) return 0;
+  if (heads <= 0 || groups <= 0 || heads % groups || n_state <= 0 || n_state > 256 || vdim <= 0 || heads > 65535 || n_entries > 65535)
+    return PK_BAD;
+  const dim3 grid(ceil_div(vdim, kRecCols), heads, n_entries);
+  bool ok = true;
+  const bool known = by_dtype(dtype, [&](auto* t) {
+    using A = std::remove_pointer_t<decltype(t)>;
+    ok = by_slices(n_state, [&](auto ns) {
+      ssd_scan_kernel<decltype(ns)::value, A><<<grid, 256, 0, as_stream(stream)>>>(
+          xbc, xbc_stride, static_cast<const A*>(proj), proj_stride, dt_off, static_cast<const A*>(A_log),
+          static_cast<const A*>(dt_bias), static_cast<const A*>(D), state, slot_stride, o, heads, groups, n_state, vdim, entry_row0,
+          entry_slot);
+    });
+  });
+  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
+}

@@ -9,6 +9,11 @@
 //   head_rms_gate_kernel    per-head RMS norm of a read-out * weight * silu / sigmoid gate * constant
 //   scalar_rms_add_kernel   residual sum with a constant factor (+ bias, + extra rows, + one extra vector), then an RMS norm
 //                           whose gain is a single number
+//   terms_rms_add_kernel    residual sum of up to three sublayer outputs, each optionally RMS-normed with a weight first, then
+//                           the RMS norm (a weight per channel) of what reads the stream next: one launch closes a layer whose
+//                           sublayers all read the same normed input, and opens the next
+//   glu_rows_kernel         act(gate) * up from two column ranges of a wider row (silu, relu or tanh-gelu)
+//   softcap_rows_kernel     cap * tanh(x / cap) on fp32 rows
 #include <algorithm>
 
 #include "common.h"
@@ -23,20 +28,23 @@ __global__ __launch_bounds__(256) void time_conv_kernel(const I* __restrict__ in
                                                         O* __restrict__ out, int64_t out_stride, int C, int K, int mode,
                                                         const int32_t* __restrict__ row_entry,
                                                         const int32_t* __restrict__ entry_row0,
-                                                        const int32_t* __restrict__ entry_slot) {
+                                                        const int32_t* __restrict__ entry_slot,
+                                                        const W* __restrict__ in_bias, const W* __restrict__ out_bias) {
   const int row = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int e = row_entry[row], r0 = entry_row0[e];
   const int local = row - r0;
   const float* tail = state + (int64_t)entry_slot[e] * slot_stride;
+  const float ib = in_bias ? ld(in_bias + c) : 0.f;   // part of every real input (the carried inputs hold it already)
   float acc = 0.f;
   for (int j = 0; j < K; ++j) {
     const int src = local - (K - 1) + j;   // row of the entry this tap reads; negative = carried from earlier steps
-    const float v = src >= 0 ? ld(in + (int64_t)(r0 + src) * in_stride + c) : tail[(int64_t)(K - 1 + src) * C + c];
+    const float v = src >= 0 ? ld(in + (int64_t)(r0 + src) * in_stride + c) + ib : tail[(int64_t)(K - 1 + src) * C + c];
     acc = fmaf(ld(w + (int64_t)c * K + j), v, acc);
   }
-  if (mode & 1) acc += ld(in + (int64_t)row * in_stride + c);
+  if (mode & 1) acc += ld(in + (int64_t)row * in_stride + c) + ib;
+  if (out_bias) acc += ld(out_bias + c);
   if (mode & 2) acc = silu_f(acc);
   st(out + (int64_t)row * out_stride + c, acc);
 }
@@ -53,9 +61,11 @@ __global__ __launch_bounds__(256) void time_conv_window_kernel(const I* __restri
                                                                int C, int K, int mode, int n_rows,
                                                                const int32_t* __restrict__ row_entry,
                                                                const int32_t* __restrict__ entry_row0,
-                                                               const int32_t* __restrict__ entry_slot) {
+                                                               const int32_t* __restrict__ entry_slot,
+                                                               const W* __restrict__ in_bias, const W* __restrict__ out_bias) {
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
+  const float ib = in_bias ? ld(in_bias + c) : 0.f, ob = out_bias ? ld(out_bias + c) : 0.f;
   float wr[KMAX], win[KMAX];
 #pragma unroll
   for (int j = 0; j < KMAX; ++j) {
@@ -75,17 +85,18 @@ __global__ __launch_bounds__(256) void time_conv_window_kernel(const I* __restri
       for (int j = 0; j < KMAX - 1; ++j) {
         const int t = KMAX - 1 - j;
         const int src = local - t;
-        win[j + 1] = t >= K ? 0.f : src >= 0 ? ld(in + (int64_t)(r0 + src) * in_stride + c) : tail[(int64_t)(K - 1 + src) * C + c];
+        win[j + 1] = t >= K ? 0.f : src >= 0 ? ld(in + (int64_t)(r0 + src) * in_stride + c) + ib : tail[(int64_t)(K - 1 + src) * C + c];
       }
     }
 #pragma unroll
     for (int j = 0; j < KMAX - 1; ++j) win[j] = win[j + 1];
-    const float cur = ld(in + (int64_t)row * in_stride + c);
+    const float cur = ld(in + (int64_t)row * in_stride + c) + ib;
     win[KMAX - 1] = cur;
     float acc = 0.f;
 #pragma unroll
     for (int j = 0; j < KMAX; ++j) acc = fmaf(wr[j], win[j], acc);
     if (mode & 1) acc += cur;
+    acc += ob;
     if (mode & 2) acc = silu_f(acc);
     st(out + (int64_t)row * out_stride + c, acc);
   }
@@ -97,12 +108,13 @@ template <typename I, typename W, typename O>
 __global__ __launch_bounds__(256) void time_conv_step_kernel(const I* __restrict__ in, int64_t in_stride, const W* __restrict__ w,
                                                              float* __restrict__ state, int64_t slot_stride, O* __restrict__ out,
                                                              int64_t out_stride, int C, int K, int mode,
-                                                             const int32_t* __restrict__ entry_slot) {
+                                                             const int32_t* __restrict__ entry_slot,
+                                                             const W* __restrict__ in_bias, const W* __restrict__ out_bias) {
   const int e = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   float* tail = state + (int64_t)entry_slot[e] * slot_stride;
-  const float cur = ld(in + (int64_t)e * in_stride + c);
+  const float cur = ld(in + (int64_t)e * in_stride + c) + (in_bias ? ld(in_bias + c) : 0.f);
   float acc = 0.f;
   for (int j = 0; j < K - 1; ++j) {
     const float v = tail[(int64_t)j * C + c];
@@ -112,23 +124,26 @@ __global__ __launch_bounds__(256) void time_conv_step_kernel(const I* __restrict
   acc = fmaf(ld(w + (int64_t)c * K + K - 1), cur, acc);
   if (K > 1) tail[(int64_t)(K - 2) * C + c] = cur;
   if (mode & 1) acc += cur;
+  if (out_bias) acc += ld(out_bias + c);
   if (mode & 2) acc = silu_f(acc);
   st(out + (int64_t)e * out_stride + c, acc);
 }
 
-template <typename I>
+template <typename I, typename W>
 __global__ __launch_bounds__(256) void time_conv_commit_kernel(const I* __restrict__ in, int64_t in_stride,
                                                                float* __restrict__ state, int64_t slot_stride, int C, int K,
                                                                const int32_t* __restrict__ entry_row0,
-                                                               const int32_t* __restrict__ entry_slot) {
+                                                               const int32_t* __restrict__ entry_slot,
+                                                               const W* __restrict__ in_bias) {
   const int e = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (c >= C) return;
+  const float ib = in_bias ? ld(in_bias + c) : 0.f;
   const int r0 = entry_row0[e], len = entry_row0[e + 1] - r0;
   float* tail = state + (int64_t)entry_slot[e] * slot_stride;
   for (int s = 0; s < K - 1; ++s) {
     const int idx = len + s;   // position in [old state (K - 1) ; this step's inputs (len)]
-    tail[(int64_t)s * C + c] = idx < K - 1 ? tail[(int64_t)idx * C + c] : ld(in + (int64_t)(r0 + idx - (K - 1)) * in_stride + c);
+    tail[(int64_t)s * C + c] = idx < K - 1 ? tail[(int64_t)idx * C + c] : ld(in + (int64_t)(r0 + idx - (K - 1)) * in_stride + c) + ib;
   }
 }
 
@@ -228,21 +243,26 @@ template <typename A>
 __global__ __launch_bounds__(256) void head_rms_gate_kernel(const float* __restrict__ o, const A* __restrict__ w, int w_per_head,
                                                             const A* __restrict__ gate, int64_t gate_stride, int gate_kind,
                                                             float factor, float eps, A* __restrict__ out, int64_t out_stride,
-                                                            int heads, int vdim, int rows) {
+                                                            int heads, int vdim, int rows, int gate_first) {
   const int64_t rh = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (rh >= (int64_t)rows * heads) return;
   const int row = (int)(rh / heads), h = (int)(rh % heads);
   const float* p = o + ((int64_t)row * heads + h) * vdim;
+  const A* gr = gate + (int64_t)row * gate_stride + (int64_t)h * vdim;
+  auto act = [&](int i) {
+    const float z = ld(gr + i);
+    return gate_kind == 0 ? silu_f(z) : sigmoid_f(z);
+  };
   float ss = 0.f;
-  for (int i = lane; i < vdim; i += 64) ss = fmaf(p[i], p[i], ss);
+  for (int i = lane; i < vdim; i += 64) {
+    const float v = gate_first ? p[i] * act(i) : p[i];   // gate_first: the gated values are what is normed
+    ss = fmaf(v, v, ss);
+  }
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
-  for (int i = lane; i < vdim; i += 64) {
-    const float z = ld(gate + (int64_t)row * gate_stride + h * vdim + i);
-    const float a = gate_kind == 0 ? silu_f(z) : sigmoid_f(z);
-    st(out + (int64_t)row * out_stride + h * vdim + i, p[i] * inv * ld(w + (w_per_head ? h * vdim : 0) + i) * a * factor);
-  }
+  for (int i = lane; i < vdim; i += 64)
+    st(out + (int64_t)row * out_stride + h * vdim + i, p[i] * act(i) * inv * ld(w + (w_per_head ? h * vdim : 0) + i) * factor);
 }
 
 // Residual sum with a constant factor, then an RMS norm whose gain is ONE number:
@@ -301,6 +321,101 @@ __global__ __launch_bounds__(256) void scalar_rms_add_kernel(const float* x_in, 
   }
 }
 
+
+// Up to three sublayer outputs join the stream at once; a term with a weight is RMS-normed over the row first:
+//   term_t = (w_t ? (y_t + bias_t) / sqrt(mean((y_t + bias_t)^2) + eps) * w_t : y_t + bias_t) * factor_t
+//   r = x_in + sum_t term_t                                  -> x_out (fp32; may alias x_in)
+//   n = r / sqrt(mean(r^2) + eps) * gain                     -> n_out (N: float or the storage type; optional)
+// NPT: values a thread keeps between the sum and the norm (d <= 256 * NPT), 0 = any d (the row is summed a second time).
+struct SumTerm { const void* y; int64_t stride; const void* bias; const void* w; float factor; };
+struct SumTerms { SumTerm t[3]; int n; };
+template <typename A, typename N, int NPT>
+__global__ __launch_bounds__(256) void terms_rms_add_kernel(const float* x_in, SumTerms terms, float* x_out,
+                                                            const A* __restrict__ gain, float eps, N* __restrict__ n_out, int d) {
+  __shared__ float red[4];
+  const int row = blockIdx.x;
+  const int64_t base = (int64_t)row * d;
+  float inv[3] = {1.f, 1.f, 1.f};
+#pragma unroll
+  for (int t = 0; t < 3; ++t) {
+    if (t >= terms.n || !terms.t[t].w) continue;     // uniform over the workgroup
+    const A* y = static_cast<const A*>(terms.t[t].y) + (int64_t)row * terms.t[t].stride;
+    const A* b = static_cast<const A*>(terms.t[t].bias);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += 256) {
+      const float v = ld(y + i) + (b ? ld(b + i) : 0.f);
+      ss = fmaf(v, v, ss);
+    }
+    inv[t] = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)d + eps);
+  }
+  auto value = [&](int i) {
+    float r = x_in ? x_in[base + i] : 0.f;
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      if (t >= terms.n) continue;
+      const A* y = static_cast<const A*>(terms.t[t].y) + (int64_t)row * terms.t[t].stride;
+      const A* b = static_cast<const A*>(terms.t[t].bias);
+      const A* w = static_cast<const A*>(terms.t[t].w);
+      float v = ld(y + i) + (b ? ld(b + i) : 0.f);
+      if (w) v = v * inv[t] * ld(w + i);
+      r = fmaf(terms.t[t].factor, v, r);
+    }
+    return r;
+  };
+  float ss = 0.f;
+  if constexpr (NPT > 0) {
+    float keep[NPT];
+#pragma unroll
+    for (int k = 0; k < NPT; ++k) {
+      const int i = threadIdx.x + 256 * k;
+      keep[k] = i < d ? value(i) : 0.f;
+      ss = fmaf(keep[k], keep[k], ss);
+    }
+    ss = block_sum<4>(ss, red);
+    const float sc = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int k = 0; k < NPT; ++k) {
+      const int i = threadIdx.x + 256 * k;
+      if (i < d) {
+        if (x_out) x_out[base + i] = keep[k];
+        if (n_out) st(n_out + base + i, keep[k] * sc * ld(gain + i));
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < d; i += 256) {
+      const float r = value(i);
+      ss = fmaf(r, r, ss);
+    }
+    ss = block_sum<4>(ss, red);   // its barriers also order every read of x_in before the writes below
+    const float sc = 1.0f / sqrtf(ss / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += 256) {
+      const float r = value(i);
+      if (x_out) x_out[base + i] = r;
+      if (n_out) st(n_out + base + i, r * sc * ld(gain + i));
+    }
+  }
+}
+
+// out[row, i] = act(gate[row, i]) * up[row, i]; gate and up are column ranges of rows with one stride
+template <typename A>
+__global__ __launch_bounds__(256) void glu_rows_kernel(const A* __restrict__ gate, const A* __restrict__ up, int64_t in_stride,
+                                                       A* __restrict__ out, int64_t out_stride, int I, int act) {
+  const int row = blockIdx.x;
+  const int i = blockIdx.y * 256 + threadIdx.x;
+  if (i >= I) return;
+  const float g = ld(gate + (int64_t)row * in_stride + i), u = ld(up + (int64_t)row * in_stride + i);
+  float a;
+  if (act == 0) a = silu_f(g);
+  else if (act == 1) a = fmaxf(g, 0.f);
+  else a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  st(out + (int64_t)row * out_stride + i, a * u);
+}
+
+__global__ __launch_bounds__(256) void softcap_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t n, float cap) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = cap * tanhf(in[i] / cap);
+}
+
 }  // namespace pk
 
 extern "C" {
@@ -308,11 +423,72 @@ using namespace pk;
 
 #define PK_BAD ((pegainfer_status_t)hipErrorInvalidValue)
 
+pegainfer_status_t pegainfer_terms_rms_add(const float* x_in, const pegainfer_sum_term* terms, int32_t n_terms, float* x_out,
+                                           const void* gain, float eps, void* n_out, int32_t n_dtype, int32_t d, int32_t rows,
+                                           int32_t dtype, pegainfer_stream_t stream) {
+  if (rows <= 0) return 0;
+  if (d <= 0 || n_terms < 0 || n_terms > 3 || (n_terms > 0 && !terms) || (!x_in && n_terms == 0) || (!x_out && !n_out) ||
+      (n_out && !gain))
+    return PK_BAD;
+  SumTerms st_{};
+  st_.n = n_terms;
+  for (int t = 0; t < n_terms; ++t) {
+    if (!terms[t].y) return PK_BAD;
+    st_.t[t] = SumTerm{terms[t].y, terms[t].y_row_stride, terms[t].bias, terms[t].norm_w, terms[t].factor};
+  }
+  bool ok = true;
+  const bool known = by_dtype(dtype, [&](auto* ta) {
+    using A = std::remove_pointer_t<decltype(ta)>;
+    ok = by_dtype(n_out ? n_dtype : dtype, [&](auto* tn) {
+      using N = std::remove_pointer_t<decltype(tn)>;
+      auto go = [&](auto npt) {
+        terms_rms_add_kernel<A, N, decltype(npt)::value><<<rows, 256, 0, as_stream(stream)>>>(
+            x_in, st_, x_out, static_cast<const A*>(gain), eps, static_cast<N*>(n_out), d);
+      };
+      if (d <= 1024) go(std::integral_constant<int, 4>());
+      else if (d <= 4096) go(std::integral_constant<int, 16>());
+      else if (d <= 8192) go(std::integral_constant<int, 32>());
+      else go(std::integral_constant<int, 0>());
+    });
+  });
+  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
+}
+
+pegainfer_status_t pegainfer_glu_rows(const void* gate, const void* up, int64_t in_row_stride, void* out, int64_t out_row_stride,
+                                      int32_t I, int32_t rows, int32_t act, int32_t dtype, pegainfer_stream_t stream) {
+  if (rows <= 0 || I <= 0) return 0;
+  if (act < 0 || act > 2) return PK_BAD;
+  const dim3 grid(rows, ceil_div(I, 256));
+  if (!by_dtype(dtype, [&](auto* t) {
+        using A = std::remove_pointer_t<decltype(t)>;
+        glu_rows_kernel<A><<<grid, 256, 0, as_stream(stream)>>>(static_cast<const A*>(gate), static_cast<const A*>(up), in_row_stride,
+                                                                static_cast<A*>(out), out_row_stride, I, act);
+      }))
+    return PK_BAD;
+  return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_softcap_rows(const float* in, float* out, int64_t n, float cap, pegainfer_stream_t stream) {
+  if (n <= 0) return 0;
+  if (!(cap > 0.f)) return PK_BAD;
+  softcap_rows_kernel<<<ceil_div(n, 256), 256, 0, as_stream(stream)>>>(in, out, n, cap);
+  return (pegainfer_status_t)hipGetLastError();
+}
+
 pegainfer_status_t pegainfer_time_conv(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w, int32_t w_dtype,
                                        const float* state, int64_t slot_stride, void* out, int32_t out_dtype,
                                        int64_t out_row_stride, int32_t channels, int32_t taps, int32_t mode,
                                        const int32_t* row_entry, const int32_t* entry_row0, const int32_t* entry_slot,
                                        int32_t n_rows, pegainfer_stream_t stream) {
+  return pegainfer_time_conv_biased(in, in_dtype, in_row_stride, w, w_dtype, nullptr, nullptr, state, slot_stride, out, out_dtype,
+                                    out_row_stride, channels, taps, mode, row_entry, entry_row0, entry_slot, n_rows, stream);
+}
+
+pegainfer_status_t pegainfer_time_conv_biased(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w, int32_t w_dtype,
+                                              const void* in_bias, const void* out_bias, const float* state, int64_t slot_stride,
+                                              void* out, int32_t out_dtype, int64_t out_row_stride, int32_t channels, int32_t taps,
+                                              int32_t mode, const int32_t* row_entry, const int32_t* entry_row0,
+                                              const int32_t* entry_slot, int32_t n_rows, pegainfer_stream_t stream) {
   if (n_rows <= 0) return 0;
   if (channels <= 0 || taps < 1) return PK_BAD;
   const dim3 grid(n_rows, ceil_div(channels, 256));
@@ -327,15 +503,18 @@ pegainfer_status_t pegainfer_time_conv(const void* in, int32_t in_dtype, int64_t
                   if (n_rows >= 4 * kConvRows && taps <= 4)
                     time_conv_window_kernel<I, W, O, 4><<<wgrid, 256, 0, as_stream(stream)>>>(
                         static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
-                        static_cast<O*>(out), out_row_stride, channels, taps, mode, n_rows, row_entry, entry_row0, entry_slot);
+                        static_cast<O*>(out), out_row_stride, channels, taps, mode, n_rows, row_entry, entry_row0, entry_slot,
+                        static_cast<const W*>(in_bias), static_cast<const W*>(out_bias));
                   else if (n_rows >= 4 * kConvRows && taps <= 8)
                     time_conv_window_kernel<I, W, O, 8><<<wgrid, 256, 0, as_stream(stream)>>>(
                         static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
-                        static_cast<O*>(out), out_row_stride, channels, taps, mode, n_rows, row_entry, entry_row0, entry_slot);
+                        static_cast<O*>(out), out_row_stride, channels, taps, mode, n_rows, row_entry, entry_row0, entry_slot,
+                        static_cast<const W*>(in_bias), static_cast<const W*>(out_bias));
                   else
                     time_conv_kernel<I, W, O><<<grid, 256, 0, as_stream(stream)>>>(
                         static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
-                        static_cast<O*>(out), out_row_stride, channels, taps, mode, row_entry, entry_row0, entry_slot);
+                        static_cast<O*>(out), out_row_stride, channels, taps, mode, row_entry, entry_row0, entry_slot,
+                        static_cast<const W*>(in_bias), static_cast<const W*>(out_bias));
                 }) && ok;
          }) && ok;
   });
@@ -346,6 +525,15 @@ pegainfer_status_t pegainfer_time_conv_step(const void* in, int32_t in_dtype, in
                                             float* state, int64_t slot_stride, void* out, int32_t out_dtype, int64_t out_row_stride,
                                             int32_t channels, int32_t taps, int32_t mode, const int32_t* entry_slot,
                                             int32_t n_entries, pegainfer_stream_t stream) {
+  return pegainfer_time_conv_step_biased(in, in_dtype, in_row_stride, w, w_dtype, nullptr, nullptr, state, slot_stride, out, out_dtype,
+                                         out_row_stride, channels, taps, mode, entry_slot, n_entries, stream);
+}
+
+pegainfer_status_t pegainfer_time_conv_step_biased(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w,
+                                                   int32_t w_dtype, const void* in_bias, const void* out_bias, float* state,
+                                                   int64_t slot_stride, void* out, int32_t out_dtype, int64_t out_row_stride,
+                                                   int32_t channels, int32_t taps, int32_t mode, const int32_t* entry_slot,
+                                                   int32_t n_entries, pegainfer_stream_t stream) {
   if (n_entries <= 0) return 0;
   if (channels <= 0 || taps < 1) return PK_BAD;
   const dim3 grid(n_entries, ceil_div(channels, 256));
@@ -358,7 +546,8 @@ pegainfer_status_t pegainfer_time_conv_step(const void* in, int32_t in_dtype, in
                   using O = std::remove_pointer_t<decltype(to)>;
                   time_conv_step_kernel<I, W, O><<<grid, 256, 0, as_stream(stream)>>>(
                       static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
-                      static_cast<O*>(out), out_row_stride, channels, taps, mode, entry_slot);
+                      static_cast<O*>(out), out_row_stride, channels, taps, mode, entry_slot, static_cast<const W*>(in_bias),
+                      static_cast<const W*>(out_bias));
                 }) && ok;
          }) && ok;
   });
@@ -368,15 +557,27 @@ pegainfer_status_t pegainfer_time_conv_step(const void* in, int32_t in_dtype, in
 pegainfer_status_t pegainfer_time_conv_commit(const void* in, int32_t in_dtype, int64_t in_row_stride, float* state,
                                               int64_t slot_stride, int32_t channels, int32_t taps, const int32_t* entry_row0,
                                               const int32_t* entry_slot, int32_t n_entries, pegainfer_stream_t stream) {
+  return pegainfer_time_conv_commit_biased(in, in_dtype, in_row_stride, nullptr, in_dtype, state, slot_stride, channels, taps, entry_row0,
+                                           entry_slot, n_entries, stream);
+}
+
+pegainfer_status_t pegainfer_time_conv_commit_biased(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* in_bias,
+                                                     int32_t bias_dtype, float* state, int64_t slot_stride, int32_t channels,
+                                                     int32_t taps, const int32_t* entry_row0, const int32_t* entry_slot,
+                                                     int32_t n_entries, pegainfer_stream_t stream) {
   if (n_entries <= 0 || taps <= 1) return 0;
   const dim3 grid(ceil_div(channels, 256), n_entries);
-  if (!by_dtype(in_dtype, [&](auto* ti) {
-        using I = std::remove_pointer_t<decltype(ti)>;
-        time_conv_commit_kernel<I><<<grid, 256, 0, as_stream(stream)>>>(static_cast<const I*>(in), in_row_stride, state,
-                                                                        slot_stride, channels, taps, entry_row0, entry_slot);
-      }))
-    return PK_BAD;
-  return (pegainfer_status_t)hipGetLastError();
+  bool ok = true;
+  const bool known = by_dtype(in_dtype, [&](auto* ti) {
+    using I = std::remove_pointer_t<decltype(ti)>;
+    ok = by_dtype(bias_dtype, [&](auto* tw) {
+      using W = std::remove_pointer_t<decltype(tw)>;
+      time_conv_commit_kernel<I, W><<<grid, 256, 0, as_stream(stream)>>>(static_cast<const I*>(in), in_row_stride, state, slot_stride,
+                                                                         channels, taps, entry_row0, entry_slot,
+                                                                         static_cast<const W*>(in_bias));
+    });
+  });
+  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
 }
 
 pegainfer_status_t pegainfer_group_rms_add(const float* x_in, const void* y, int32_t y_dtype, const void* w, int32_t groups,
@@ -424,6 +625,14 @@ pegainfer_status_t pegainfer_head_rms_gate(const float* o, const void* w, int32_
                                            int64_t gate_stride, int32_t gate_kind, float factor, float eps, void* out,
                                            int64_t out_stride, int32_t heads, int32_t vdim, int32_t rows, int32_t dtype,
                                            pegainfer_stream_t stream) {
+  return pegainfer_head_gate_rms(o, w, w_per_head, gate, gate_stride, gate_kind, 0, factor, eps, out, out_stride, heads, vdim, rows,
+                                 dtype, stream);
+}
+
+pegainfer_status_t pegainfer_head_gate_rms(const float* o, const void* w, int32_t w_per_head, const void* gate, int64_t gate_stride,
+                                           int32_t gate_kind, int32_t gate_first, float factor, float eps, void* out,
+                                           int64_t out_stride, int32_t heads, int32_t vdim, int32_t rows, int32_t dtype,
+                                           pegainfer_stream_t stream) {
   if (rows <= 0) return 0;
   if (heads <= 0 || vdim <= 0) return PK_BAD;
   const int blocks = ceil_div((long)rows * heads, 4);
@@ -432,7 +641,7 @@ pegainfer_status_t pegainfer_head_rms_gate(const float* o, const void* w, int32_
         head_rms_gate_kernel<A><<<blocks, 256, 0, as_stream(stream)>>>(o, static_cast<const A*>(w), w_per_head,
                                                                        static_cast<const A*>(gate), gate_stride, gate_kind,
                                                                        factor, eps, static_cast<A*>(out), out_stride, heads,
-                                                                       vdim, rows);
+                                                                       vdim, rows, gate_first);
       }))
     return PK_BAD;
   return (pegainfer_status_t)hipGetLastError();

@@ -20,7 +20,7 @@ _SCALARS = {
     "int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "uint32_t": ctypes.c_uint32,
     "uint64_t": ctypes.c_uint64, "float": ctypes.c_float, "int": ctypes.c_int,
     "pegainfer_stream_t": ctypes.c_void_p, "pegainfer_status_t": ctypes.c_int32,
-    "pegainfer_qwen3_t": ctypes.c_void_p, "pegainfer_qwen35_t": ctypes.c_void_p, "pegainfer_duguzen_t": ctypes.c_void_p, "pegainfer_feruzen_t": ctypes.c_void_p, "pegainfer_ramalix_t": ctypes.c_void_p, "size_t": ctypes.c_size_t,
+    "pegainfer_qwen3_t": ctypes.c_void_p, "pegainfer_qwen35_t": ctypes.c_void_p, "pegainfer_duguzen_t": ctypes.c_void_p, "pegainfer_feruzen_t": ctypes.c_void_p, "pegainfer_ramalix_t": ctypes.c_void_p, "pegainfer_kukulorn_t": ctypes.c_void_p, "size_t": ctypes.c_size_t,
     "pegainfer_sched_t": ctypes.c_void_p, "pegainfer_comm_t": ctypes.c_void_p, "pegainfer_ep_hub_t": ctypes.c_void_p,
     "pegainfer_ep_t": ctypes.c_void_p,
     "double": ctypes.c_double,
@@ -110,10 +110,10 @@ def lib():
 
 
 def host_lib():
-    """libpegainfer_qwen3.so (include/pegainfer_qwen3.h, pegainfer_qwen35.h, pegainfer_duguzen.h, pegainfer_feruzen.h, pegainfer_ramalix.h, pegainfer_scheduler.h,
+    """libpegainfer_qwen3.so (include/pegainfer_qwen3.h, pegainfer_qwen35.h, pegainfer_duguzen.h, pegainfer_feruzen.h, pegainfer_ramalix.h, pegainfer_kukulorn.h, pegainfer_scheduler.h,
     pegainfer_comm.h)."""
     if "h" not in _cache:
         lib()
         _cache["h"] = _Lib("libpegainfer_qwen3.so", "pegainfer_qwen3.h", "pegainfer_qwen35.h", "pegainfer_scheduler.h",
-                           "pegainfer_comm.h", "pegainfer_duguzen.h", "pegainfer_feruzen.h", "pegainfer_ramalix.h")
+                           "pegainfer_comm.h", "pegainfer_duguzen.h", "pegainfer_feruzen.h", "pegainfer_ramalix.h", "pegainfer_kukulorn.h")
     return _cache["h"]

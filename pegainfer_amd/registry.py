@@ -1,7 +1,7 @@
 """Model registry: which engine serves a model folder, decided by its config.json.
 
 Hugging Face style configurations name their family in ``model_type`` / ``architectures`` (Qwen3, Qwen3.5); Duguzen,
-Feruzen and Ramalix name it in ``architecture``.  ``load_engine`` builds the engine with the weights of the folder; ``scheduler_for`` puts the
+Feruzen, Ramalix and Kukulorn name it in ``architecture``.  ``load_engine`` builds the engine with the weights of the folder; ``scheduler_for`` puts the
 continuous-batching scheduler (include/pegainfer_scheduler.h) on top of it.
 """
 import json
@@ -41,6 +41,12 @@ def _ramalix(model_dir, cfg, **kw):
                                          dtype=kw.get("dtype", "bfloat16"), device=kw.get("device", 0))
 
 
+def _kukulorn(model_dir, cfg, **kw):
+    from .kukulorn import KukulornEngine
+    return KukulornEngine.from_pretrained(model_dir, max_tokens=kw.get("max_tokens", 4096), max_requests=kw.get("max_requests", 8),
+                                          dtype=kw.get("dtype", "bfloat16"), device=kw.get("device", 0))
+
+
 # family -> (loader, dtypes it can be served in)
 REGISTRY = {
     "qwen3": (_qwen3, ("bfloat16",)),
@@ -48,12 +54,13 @@ REGISTRY = {
     "duguzen": (_duguzen, ("bfloat16", "float32")),
     "feruzen": (_feruzen, ("bfloat16", "float32")),
     "ramalix": (_ramalix, ("bfloat16", "float32")),
+    "kukulorn": (_kukulorn, ("bfloat16", "float32")),
 }
 
 
 def family_of(cfg):
     """the registry key of a parsed config.json, or None"""
-    if str(cfg.get("architecture", "")).lower() in ("duguzen", "feruzen", "ramalix"):
+    if str(cfg.get("architecture", "")).lower() in ("duguzen", "feruzen", "ramalix", "kukulorn"):
         return str(cfg["architecture"]).lower()
     names = [str(cfg.get("model_type", ""))] + [str(a) for a in cfg.get("architectures", [])]
     low = " ".join(names).lower()

@@ -60,7 +60,8 @@ class Scheduler:
         create = {"Qwen35Engine": lib.pegainfer_sched_create_qwen35,
                   "DuguzenEngine": lib.pegainfer_sched_create_duguzen,
                   "FeruzenEngine": lib.pegainfer_sched_create_feruzen,
-                  "RamalixEngine": lib.pegainfer_sched_create_ramalix}.get(type(engine).__name__, lib.pegainfer_sched_create_qwen3)
+                  "RamalixEngine": lib.pegainfer_sched_create_ramalix,
+                  "KukulornEngine": lib.pegainfer_sched_create_kukulorn}.get(type(engine).__name__, lib.pegainfer_sched_create_qwen3)
         h = create(engine.h, seed, st.ctypes.data if st.size else None, int(st.size))
         return cls(h, keep=engine)
 
