@@ -177,23 +177,24 @@ class Ragged:
         self.entry_row0, self.entry_slot, self.row_entry, self.positions = i32(row0), i32(slots), i32(ent), i32(pos)
 
 
-def time_conv(x, w, state, rg, residual=False, silu=False, out_dtype=None, channels=None):
-    """causal per-channel convolution over time; state fp32 [slots, taps - 1, C] is read, then moved on by the step's rows"""
+def time_conv(x, w, state, rg, residual=False, silu=False, out_dtype=None, channels=None, in_bias=None, out_bias=None):
+    """causal per-channel convolution over time; state fp32 [slots, taps - 1, C] is read, then moved on by the step's rows.
+    in_bias [C] joins every real input (and so the carried ones), out_bias [C] the sum before the activation; both in w's type"""
     C = channels or w.shape[0]
     taps = w.shape[1]
     out = torch.empty((x.shape[0], C), dtype=out_dtype or x.dtype, device=x.device)
     slot_stride = state.shape[1] * state.shape[2] if state.dim() == 3 else 0
     L = ffi.lib()
     if all(n == 1 for n in rg.lens):      # decoding: output and the moved-on tail in one launch
-        _chk(L.pegainfer_time_conv_step(_p(x), _dt(x), x.stride(0), _p(w), _dt(w), _p(state), slot_stride, _p(out), _dt(out), C, C,
-                                        taps, (1 if residual else 0) | (2 if silu else 0), _p(rg.entry_slot), rg.n, _stream()),
-             "time_conv_step")
+        _chk(L.pegainfer_time_conv_step_biased(_p(x), _dt(x), x.stride(0), _p(w), _dt(w), _p(in_bias), _p(out_bias), _p(state),
+                                               slot_stride, _p(out), _dt(out), C, C, taps, (1 if residual else 0) | (2 if silu else 0),
+                                               _p(rg.entry_slot), rg.n, _stream()), "time_conv_step")
         return out
-    _chk(L.pegainfer_time_conv(_p(x), _dt(x), x.stride(0), _p(w), _dt(w), _p(state), slot_stride, _p(out), _dt(out), C, C, taps,
-                               (1 if residual else 0) | (2 if silu else 0), _p(rg.row_entry), _p(rg.entry_row0),
-                               _p(rg.entry_slot), x.shape[0], _stream()), "time_conv")
-    _chk(L.pegainfer_time_conv_commit(_p(x), _dt(x), x.stride(0), _p(state), slot_stride, C, taps, _p(rg.entry_row0),
-                                      _p(rg.entry_slot), rg.n, _stream()), "time_conv_commit")
+    _chk(L.pegainfer_time_conv_biased(_p(x), _dt(x), x.stride(0), _p(w), _dt(w), _p(in_bias), _p(out_bias), _p(state), slot_stride,
+                                      _p(out), _dt(out), C, C, taps, (1 if residual else 0) | (2 if silu else 0), _p(rg.row_entry),
+                                      _p(rg.entry_row0), _p(rg.entry_slot), x.shape[0], _stream()), "time_conv")
+    _chk(L.pegainfer_time_conv_commit_biased(_p(x), _dt(x), x.stride(0), _p(in_bias), _dt(w), _p(state), slot_stride, C, taps,
+                                             _p(rg.entry_row0), _p(rg.entry_slot), rg.n, _stream()), "time_conv_commit")
     return out
 
 
@@ -399,3 +400,100 @@ def route_combine_gated(y_pairs, weight, add, add_gate_f32, out_dtype):
                                                  0 if add_gate_f32 is None else add_gate_f32.stride(0), _p(out), d, top, rows,
                                                  _dt(out), _stream()), "route_combine_gated")
     return out
+
+
+# ---- several sublayers behind one norm, attention with shaped scores and gates, state-space scan ----
+class SumTerm(ctypes.Structure):
+    _fields_ = [("y", ctypes.c_void_p), ("y_row_stride", ctypes.c_int64), ("bias", ctypes.c_void_p), ("norm_w", ctypes.c_void_p),
+                ("factor", ctypes.c_float)]
+
+
+def terms_rms_add(x, terms, gain=None, eps=1e-6, out_dtype=None):
+    """r = x + sum_t factor_t * (norm_w_t ? rms_norm(y_t + bias_t) * norm_w_t : y_t + bias_t);  n = rms_norm(r) * gain.
+    x fp32 [rows, d] or None; terms: up to three (y, bias or None, norm_w or None, factor); -> (r fp32, n in out_dtype or None)"""
+    ref = terms[0][0] if terms else gain
+    rows, d = (x.shape if x is not None else terms[0][0].shape)
+    arr = (SumTerm * max(1, len(terms)))()
+    for i, (y, bias, nw, f) in enumerate(terms):
+        arr[i] = SumTerm(_p(y), y.stride(0), _p(bias), _p(nw), float(f))
+    r = torch.empty((rows, d), dtype=torch.float32, device=ref.device)
+    n = torch.empty((rows, d), dtype=out_dtype or ref.dtype, device=ref.device) if gain is not None else None
+    _chk(ffi.lib().pegainfer_terms_rms_add(_p(x), ctypes.addressof(arr) if terms else None, len(terms), _p(r), _p(gain), float(eps), _p(n),
+                                           _dt(n) if n is not None else 0, d, rows, _dt(ref), _stream()), "terms_rms_add")
+    return r, n
+
+
+def glu_rows(gate, up, act="relu"):
+    """act(gate) * up; gate and up are [rows, I] views of rows with one stride (column ranges of a wider matrix)"""
+    rows, I = gate.shape
+    assert gate.stride(0) == up.stride(0)
+    out = torch.empty((rows, I), dtype=gate.dtype, device=gate.device)
+    _chk(ffi.lib().pegainfer_glu_rows(_p(gate), _p(up), gate.stride(0), _p(out), I, I, rows, {"silu": 0, "relu": 1, "gelu_tanh": 2}[act],
+                                      _dt(gate), _stream()), "glu_rows")
+    return out
+
+
+def softcap_rows(x_f32, cap):
+    out = torch.empty_like(x_f32)
+    _chk(ffi.lib().pegainfer_softcap_rows(_p(x_f32), _p(out), x_f32.numel(), float(cap), _stream()), "softcap_rows")
+    return out
+
+
+def head_gate_rms(o_f32, w, gate, gate_kind, eps, heads, vdim, gate_first=True, factor=1.0):
+    """head_rms_gate with the order chosen: gate_first norms the gated values"""
+    rows = o_f32.shape[0]
+    out = torch.empty((rows, heads * vdim), dtype=w.dtype, device=w.device)
+    _chk(ffi.lib().pegainfer_head_gate_rms(_p(o_f32), _p(w), int(w.numel() != vdim), _p(gate), gate.stride(0),
+                                           0 if gate_kind == "silu" else 1, int(bool(gate_first)), float(factor), float(eps), _p(out),
+                                           out.stride(0), heads, vdim, rows, _dt(w), _stream()), "head_gate_rms")
+    return out
+
+
+QKNORM = {"head_weight": 0, "head_unit_after": 1, "all_weight": 2}
+
+
+def qk_prep_paged_form(proj, offs, heads, kv_heads, dim, vdim, rg, page_indptr, page_ids, cache, page_stride, k_off, v_off, page_size,
+                       q_norm=None, k_norm=None, norm_kind="head_weight", eps=0.0, q_bias=None, k_bias=None, v_bias=None, inv_freq=None,
+                       rot_dims=0, halves=False):
+    """proj: rows of the cache's type or fp32 (what a convolution left); queries -> fp32 [rows, heads, dim]; keys and values -> the
+    cache entry of (request, position)"""
+    q = torch.empty((proj.shape[0], heads, dim), dtype=torch.float32, device=proj.device)
+    _chk(ffi.lib().pegainfer_qk_prep_paged_form(_p(proj), _dt(proj), proj.stride(0), offs[0], offs[1], offs[2], heads, kv_heads, dim, vdim,
+                                                _p(q_norm), _p(k_norm), QKNORM[norm_kind], float(eps), _p(q_bias), _p(k_bias), _p(v_bias),
+                                                0.0, 0, _p(inv_freq), rot_dims, int(bool(halves)), _p(rg.positions), _p(rg.row_entry),
+                                                _p(page_indptr), _p(page_ids), _p(cache), page_stride, k_off, v_off, page_size, _p(q), None,
+                                                proj.shape[0], _dt(cache), _stream()), "qk_prep_paged_form")
+    return q
+
+
+def paged_attention_masked(q, cache, page_stride, k_off, v_off, page_size, rg, page_indptr, page_ids, kv_heads, vdim, scale, softcap=0.0,
+                           window=0, keep_first=0, dist_bias=None, gate=None, gate_per_head=False, block=0, sink=None, n_split=1,
+                           plain=False):
+    """q fp32 [rows, heads, dim]; dist_bias fp32 [n_dist, heads]; gate: a view of rows in the cache's type ([rows, heads * vdim] or
+    [rows, heads])"""
+    T, H, dim = q.shape
+    out = torch.empty((T, H * vdim), dtype=cache.dtype, device=q.device)
+    t = attention_tiles(rg.lens, H // kv_heads, q.device)
+    ws = None
+    if n_split > 1:
+        ws = torch.empty(ffi.lib().pegainfer_paged_attention_workspace(t[0].numel(), kv_heads, vdim, 1, n_split), dtype=torch.float32,
+                         device=q.device)
+    _chk(ffi.lib().pegainfer_paged_attention_masked(_p(q), _p(cache), page_stride, k_off, v_off, page_size, _p(rg.positions),
+                                                    _p(rg.row_entry), _p(page_indptr), _p(page_ids), H, kv_heads, dim, vdim, float(scale),
+                                                    1.0, _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), t[0].numel(), _p(out), out.stride(0), 1,
+                                                    0.0, int(block), _p(sink), 0, 0.0, float(softcap), int(window), int(keep_first),
+                                                    _p(dist_bias), 0 if dist_bias is None else dist_bias.shape[0], _p(gate),
+                                                    0 if gate is None else gate.stride(0),
+                                                    0 if gate is None else (2 if gate_per_head else 1), int(n_split), _p(ws),
+                                                    int(bool(plain)), _dt(cache), _stream()), "paged_attention_masked")
+    return out
+
+
+def ssd_scan(xbc_f32, proj, dt_off, A_log, dt_bias, D, state, heads, groups, n_state, vdim, rg):
+    """selective state-space scan; xbc fp32 [rows, heads * vdim + 2 * groups * n_state]; proj rows (storage type) hold the raw step
+    sizes at dt_off; state fp32 [slots, heads * n_state * vdim] is read and moved on; -> y fp32 [rows, heads * vdim]"""
+    y = torch.empty((xbc_f32.shape[0], heads * vdim), dtype=torch.float32, device=proj.device)
+    _chk(ffi.lib().pegainfer_ssd_scan(_p(xbc_f32), xbc_f32.stride(0), _p(proj), proj.stride(0), dt_off, _p(A_log), _p(dt_bias), _p(D),
+                                      _p(state), state.stride(0), _p(y), heads, groups, n_state, vdim, _p(rg.entry_row0), _p(rg.entry_slot),
+                                      rg.n, _dt(proj), _stream()), "ssd_scan")
+    return y
