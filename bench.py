@@ -661,11 +661,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--ctx", type=int, default=1024, help="prompt length before the timed decode steps")
     ap.add_argument("--batch", type=int, default=1, help="requests decoded together per rank")
-    ap.add_argument("--model", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b", "qwen3.5-4b", "duguzen", "feruzen", "ramalix"],
+    ap.add_argument("--model", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b", "qwen3.5-4b", "duguzen", "feruzen", "ramalix", "kukulorn"],
                     help="duguzen: prefill / decode throughput of the Duguzen design at real layer sizes beside Qwen3 at equal size "
                          "(pegainfer_amd/bench_duguzen.py; its own JSON line, not the headline metric); feruzen: the same for the "
                          "Feruzen design beside Qwen3.5 at equal size (pegainfer_amd/bench_feruzen.py); ramalix: the Ramalix design beside "
-                         "Feruzen at equal size (pegainfer_amd/bench_ramalix.py)")
+                         "Feruzen at equal size (pegainfer_amd/bench_ramalix.py); kukulorn: the Kukulorn design beside Feruzen at "
+                         "equal size (pegainfer_amd/bench_kukulorn.py)")
     ap.add_argument("--dz-size", default="mid", choices=["small", "mid", "large", "all"], help="layer sizes of --model duguzen")
     ap.add_argument("--fz-size", default="mid", choices=["small", "mid", "large", "all"], help="layer sizes of --model feruzen")
     ap.add_argument("--fz-only", default="both", choices=["both", "feruzen", "qwen35"], help="--model feruzen: which side to run")
@@ -673,6 +674,10 @@ def main():
     ap.add_argument("--rx-only", default="both", choices=["both", "ramalix", "feruzen"], help="--model ramalix: which side to run")
     ap.add_argument("--rx-phase", default="all", choices=["all", "prefill", "decode"],
                     help="--model ramalix: prefill or decode (bs 1) alone, for a kernel trace of that phase")
+    ap.add_argument("--kk-size", default="mid", choices=["small", "mid", "large", "all"], help="layer sizes of --model kukulorn")
+    ap.add_argument("--kk-only", default="both", choices=["both", "kukulorn", "feruzen"], help="--model kukulorn: which side to run")
+    ap.add_argument("--kk-phase", default="all", choices=["all", "prefill", "decode"],
+                    help="--model kukulorn: prefill or decode (bs 1) alone, for a kernel trace of that phase")
     ap.add_argument("--decode-mode", type=int, choices=[0, 1], default=int(os.environ.get("PEGAINFER_DECODE_MODE", "1")),
                     help="0 = reference op sequence 1:1, 1 = fused MI355X decode kernels (bit-identical)")
     ap.add_argument("--split-policy", type=int, default=1)
@@ -717,6 +722,9 @@ def main():
     if args.model == "ramalix":
         from pegainfer_amd import bench_ramalix
         return bench_ramalix.run(args)
+    if args.model == "kukulorn":
+        from pegainfer_amd import bench_kukulorn
+        return bench_kukulorn.run(args)
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # plain `python bench.py --gpus N`: become the launcher - one process per GPU over RCCL, exactly what the
