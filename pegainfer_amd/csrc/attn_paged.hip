@@ -1,6 +1,6 @@
 // Softmax attention over a paged key/value cache for any head sizes and grouped key/value heads, in a bf16 and an fp32
 // storage instance; norms, angles, scores, softmax state and accumulators are fp32 in both.
-//   qk_prep_paged_kernel       one workgroup per token row, a wave per head: optional bias, optional RMS norm over the head
+//   qk_prep_paged_kernel       one or several workgroups per token row, a wave per head: optional bias, optional RMS norm over the head
 //                              (plain weight), optional position-dependent query factor (query temperature), rotation
 //                              of neighbouring pairs (2i, 2i + 1) of the first rot_dims values by position * inv_freq[i],
 //                              queries to an fp32 buffer, keys and values into the cache entry of (request, position)
@@ -64,7 +64,8 @@ __global__ __launch_bounds__(256) void qk_prep_paged_kernel(
     inv_all_k = 1.0f / sqrtf(block_sum<4>(sk, red) / (float)(G * dim) + eps);
   }
   const int half = rot_dims >> 1;
-  for (int hh = wave; hh < H + G; hh += 4) {
+  // the row's heads are dealt to the workgroups of its grid column, a wave per head
+  for (int hh = blockIdx.y * 4 + wave; hh < H + G; hh += 4 * gridDim.y) {
     const bool is_q = hh < H;
     const int hd = is_q ? hh : hh - H;
     const I* src = is_q ? pr + q_off + (int64_t)hd * dim : pr + k_off + (int64_t)hd * dim;
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(256) void qk_prep_paged_kernel(
     }
     __builtin_amdgcn_wave_barrier();
   }
-  for (int i = threadIdx.x; i < G * vdim; i += 256) {
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < G * vdim; i += 256 * gridDim.y) {
     A* dst = cache + page * page_stride + v_cache_off + (int64_t)slot * G * vdim + i;
     st(dst, ld(pr + v_off + i) + (v_bias ? ld(v_bias + i) : 0.f));
   }
@@ -448,7 +449,10 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int lo0 = attn_row_lo(form, positions[row0]);   // rows of a tile are in position order: the lowest run start
   const int kfirst = form.keep_first > 0 ? 0 : (lo0 / kAttKeys) * kAttKeys;
   // zeros everywhere first: padding columns, rows past the tile's, keys past the context's end must multiply as zeros
-  for (int i = tid; i < (kAttKeys + kAttRows) * ks + VP * kMfVs; i += 256) s_k[i] = 0;
+  {   // (the tiles' bytes are a multiple of 16: ks is a multiple of 4 values, the row counts of 16, VP * kMfVs of 8)
+    u32x4* z = reinterpret_cast<u32x4*>(smraw);
+    for (int i = tid; i < ((kAttKeys + kAttRows) * ks + VP * kMfVs) / 8; i += 256) z[i] = u32x4{0u, 0u, 0u, 0u};
+  }
   __syncthreads();
   for (int i = tid; i < nrows * qd; i += 256) {
     const int lr = i / qd, c = i % qd;
@@ -741,7 +745,9 @@ pegainfer_status_t pegainfer_qk_prep_paged_form(const void* proj, int32_t proj_d
     using A = std::remove_pointer_t<decltype(t)>;
     ok = by_dtype(proj_dtype, [&](auto* ti) {
       using I = std::remove_pointer_t<decltype(ti)>;
-      qk_prep_paged_kernel<A, I><<<n_rows, 256, (size_t)4 * dim * sizeof(float), as_stream(stream)>>>(
+      // few rows (decoding): the heads of a row spread over several workgroups, four heads each; many rows fill the chip alone
+      const int per_row = n_rows >= 512 ? 1 : std::min(16, ceil_div(heads + kv_heads, 4));
+      qk_prep_paged_kernel<A, I><<<dim3(n_rows, per_row), 256, (size_t)4 * dim * sizeof(float), as_stream(stream)>>>(
           static_cast<const I*>(proj), proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim, static_cast<const A*>(q_norm),
           static_cast<const A*>(k_norm), eps, inv_freq, rot_dims, positions, row_entry, page_indptr, page_ids, static_cast<A*>(cache),
           page_stride, k_cache_off, v_cache_off, page_size, q_out, static_cast<A*>(q_out_stored), static_cast<const A*>(q_bias),

@@ -226,11 +226,11 @@ static void mfma_form_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
 // ------------------------------------------------------------------ few-rows form (decode)
 // At most R rows per tile (a decode step's tokens, or the pairs one expert received): the weights are streamed once with
 // 16-byte loads, the rows wait in LDS as fp32, a wave owns one output at a time (lanes over k, butterfly sum), 32 outputs per
-// workgroup.  fp32 arithmetic for both storage types; the k order of an output is fixed by K alone.
-constexpr int kRowsFormOutputs = 32;
-
-template <typename TX, typename TW, typename TY, typename TG, int R>
+// workgroup - or 8 (OUT) when 32 would leave most of the chip without a workgroup (a matrix of a few thousand outputs).  fp32
+// arithmetic for both storage types; the k order of an output is fixed by K alone, whatever OUT is.
+template <typename TX, typename TW, typename TY, typename TG, int R, int OUT = 32>
 __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_desc d) {
+  constexpr int kRowsFormOutputs = OUT;
   extern __shared__ float xr[];    // [R][K]
   __shared__ int xrow[R], yrow[R];
   int g, row0, nrows;
@@ -261,8 +261,8 @@ __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_d
   __syncthreads();
   TY* Y = static_cast<TY*>(d.y) + (int64_t)g * d.y_group_stride;
   const int m_base = blockIdx.y * kRowsFormOutputs;
-  // a wave owns 8 of the workgroup's 32 outputs and walks them four at a time: four independent weight streams in flight
-  constexpr int MB = 4;
+  // a wave owns a quarter of the workgroup's outputs and walks them four at a time: four independent weight streams in flight
+  constexpr int MB = OUT >= 16 ? 4 : OUT / 4;
   for (int mg = 0; mg < kRowsFormOutputs / 4; mg += MB) {
     const int mw = m_base + wave * (kRowsFormOutputs / 4) + mg;
     if (mw >= d.m) break;
@@ -315,13 +315,19 @@ __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_d
 
 template <typename TX, typename TW, typename TY, typename TG, int R>
 static void rows_form_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
-  auto kern = &gemm_strided_rows_kernel<TX, TW, TY, TG, R>;
+  auto kern = &gemm_strided_rows_kernel<TX, TW, TY, TG, R, 32>;
+  auto kern8 = &gemm_strided_rows_kernel<TX, TW, TY, TG, R, 8>;
   // 150 KB of rows at most (checked by the caller) next to the kernel's few static words
-  static const bool once = (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                152 * 1024), true);
+  static const bool once = (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024),
+                            hipFuncSetAttribute(reinterpret_cast<const void*>(kern8), hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024),
+                            true);
   (void)once;
-  dim3 grid(d.tile_group ? d.max_tiles : ceil_div(d.rows, R), ceil_div(d.m, kRowsFormOutputs), d.tile_group ? 1 : d.groups);
-  kern<<<grid, 256, (size_t)R * d.k * sizeof(float), s>>>(d);
+  const int row_tiles = d.tile_group ? d.max_tiles : ceil_div(d.rows, R), groups = d.tile_group ? 1 : d.groups;
+  // 32 outputs per workgroup unless that leaves most compute units without one
+  const bool fine = (long)row_tiles * groups * ceil_div(d.m, 32) < device_cus();
+  dim3 grid(row_tiles, ceil_div(d.m, fine ? 8 : 32), groups);
+  if (fine) kern8<<<grid, 256, (size_t)R * d.k * sizeof(float), s>>>(d);
+  else kern<<<grid, 256, (size_t)R * d.k * sizeof(float), s>>>(d);
 }
 
 static inline bool chunks_ok(const pegainfer_gemm_desc& d) {

@@ -261,8 +261,11 @@ __global__ __launch_bounds__(256) void head_rms_gate_kernel(const float* __restr
   }
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
-  for (int i = lane; i < vdim; i += 64)
-    st(out + (int64_t)row * out_stride + h * vdim + i, p[i] * act(i) * inv * ld(w + (w_per_head ? h * vdim : 0) + i) * factor);
+  for (int i = lane; i < vdim; i += 64) {
+    const float wv = ld(w + (w_per_head ? h * vdim : 0) + i);
+    // (each order keeps its own sequence of roundings: norm, weight, gate, factor - or gate, norm, weight, factor)
+    st(out + (int64_t)row * out_stride + h * vdim + i, gate_first ? p[i] * act(i) * inv * wv * factor : p[i] * inv * wv * act(i) * factor);
+  }
 }
 
 // Residual sum with a constant factor, then an RMS norm whose gain is ONE number:
@@ -329,12 +332,17 @@ __global__ __launch_bounds__(256) void scalar_rms_add_kernel(const float* x_in, 
 // NPT: values a thread keeps between the sum and the norm (d <= 256 * NPT), 0 = any d (the row is summed a second time).
 struct SumTerm { const void* y; int64_t stride; const void* bias; const void* w; float factor; };
 struct SumTerms { SumTerm t[3]; int n; };
-template <typename A, typename N, int NPT>
+// VEC: d, the terms' strides and every pointer allow four values per load.
+template <typename A, typename N, int NPT, bool VEC>
 __global__ __launch_bounds__(256) void terms_rms_add_kernel(const float* x_in, SumTerms terms, float* x_out,
                                                             const A* __restrict__ gain, float eps, N* __restrict__ n_out, int d) {
   __shared__ float red[4];
+  constexpr int V = VEC ? 4 : 1;
   const int row = blockIdx.x;
   const int64_t base = (int64_t)row * d;
+  auto load = [&](const auto* p, float* o) {
+    if constexpr (VEC) ld4(p, o); else o[0] = ld(p);
+  };
   float inv[3] = {1.f, 1.f, 1.f};
 #pragma unroll
   for (int t = 0; t < 3; ++t) {
@@ -342,56 +350,88 @@ __global__ __launch_bounds__(256) void terms_rms_add_kernel(const float* x_in, S
     const A* y = static_cast<const A*>(terms.t[t].y) + (int64_t)row * terms.t[t].stride;
     const A* b = static_cast<const A*>(terms.t[t].bias);
     float ss = 0.f;
-    for (int i = threadIdx.x; i < d; i += 256) {
-      const float v = ld(y + i) + (b ? ld(b + i) : 0.f);
-      ss = fmaf(v, v, ss);
+    for (int i = threadIdx.x * V; i < d; i += 256 * V) {
+      float v[V], bv[V];
+      load(y + i, v);
+      if (b) load(b + i, bv);
+#pragma unroll
+      for (int u = 0; u < V; ++u) {
+        const float z = v[u] + (b ? bv[u] : 0.f);
+        ss = fmaf(z, z, ss);
+      }
     }
     inv[t] = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)d + eps);
   }
-  auto value = [&](int i) {
-    float r = x_in ? x_in[base + i] : 0.f;
+  auto value = [&](int i, float* r) {      // V values from column i on
+    if (x_in) load(x_in + base + i, r);
+    else {
+#pragma unroll
+      for (int u = 0; u < V; ++u) r[u] = 0.f;
+    }
 #pragma unroll
     for (int t = 0; t < 3; ++t) {
       if (t >= terms.n) continue;
       const A* y = static_cast<const A*>(terms.t[t].y) + (int64_t)row * terms.t[t].stride;
       const A* b = static_cast<const A*>(terms.t[t].bias);
       const A* w = static_cast<const A*>(terms.t[t].w);
-      float v = ld(y + i) + (b ? ld(b + i) : 0.f);
-      if (w) v = v * inv[t] * ld(w + i);
-      r = fmaf(terms.t[t].factor, v, r);
+      float v[V], bv[V], wv[V];
+      load(y + i, v);
+      if (b) load(b + i, bv);
+      if (w) load(w + i, wv);
+#pragma unroll
+      for (int u = 0; u < V; ++u) {
+        float z = v[u] + (b ? bv[u] : 0.f);
+        if (w) z = z * inv[t] * wv[u];
+        r[u] = fmaf(terms.t[t].factor, z, r[u]);
+      }
     }
-    return r;
+  };
+  auto store = [&](int i, const float* r, float sc) {
+    if (x_out) {
+      if constexpr (VEC) st4(x_out + base + i, r); else x_out[base + i] = r[0];
+    }
+    if (n_out) {
+      float g[V], o[V];
+      load(gain + i, g);
+#pragma unroll
+      for (int u = 0; u < V; ++u) o[u] = r[u] * sc * g[u];
+      if constexpr (VEC) st4(n_out + base + i, o); else st(n_out + base + i, o[0]);
+    }
   };
   float ss = 0.f;
   if constexpr (NPT > 0) {
     float keep[NPT];
 #pragma unroll
-    for (int k = 0; k < NPT; ++k) {
-      const int i = threadIdx.x + 256 * k;
-      keep[k] = i < d ? value(i) : 0.f;
-      ss = fmaf(keep[k], keep[k], ss);
+    for (int k = 0; k < NPT; k += V) {
+      const int i = (threadIdx.x + 256 * (k / V)) * V;
+      if (i < d) value(i, keep + k);
+      else {
+#pragma unroll
+        for (int u = 0; u < V; ++u) keep[k + u] = 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < V; ++u) ss = fmaf(keep[k + u], keep[k + u], ss);
     }
     ss = block_sum<4>(ss, red);
     const float sc = 1.0f / sqrtf(ss / (float)d + eps);
 #pragma unroll
-    for (int k = 0; k < NPT; ++k) {
-      const int i = threadIdx.x + 256 * k;
-      if (i < d) {
-        if (x_out) x_out[base + i] = keep[k];
-        if (n_out) st(n_out + base + i, keep[k] * sc * ld(gain + i));
-      }
+    for (int k = 0; k < NPT; k += V) {
+      const int i = (threadIdx.x + 256 * (k / V)) * V;
+      if (i < d) store(i, keep + k, sc);
     }
   } else {
-    for (int i = threadIdx.x; i < d; i += 256) {
-      const float r = value(i);
-      ss = fmaf(r, r, ss);
+    for (int i = threadIdx.x * V; i < d; i += 256 * V) {
+      float r[V];
+      value(i, r);
+#pragma unroll
+      for (int u = 0; u < V; ++u) ss = fmaf(r[u], r[u], ss);
     }
     ss = block_sum<4>(ss, red);   // its barriers also order every read of x_in before the writes below
     const float sc = 1.0f / sqrtf(ss / (float)d + eps);
-    for (int i = threadIdx.x; i < d; i += 256) {
-      const float r = value(i);
-      if (x_out) x_out[base + i] = r;
-      if (n_out) st(n_out + base + i, r * sc * ld(gain + i));
+    for (int i = threadIdx.x * V; i < d; i += 256 * V) {
+      float r[V];
+      value(i, r);
+      store(i, r, sc);
     }
   }
 }
@@ -441,9 +481,16 @@ pegainfer_status_t pegainfer_terms_rms_add(const float* x_in, const pegainfer_su
     using A = std::remove_pointer_t<decltype(ta)>;
     ok = by_dtype(n_out ? n_dtype : dtype, [&](auto* tn) {
       using N = std::remove_pointer_t<decltype(tn)>;
+      bool vec = d % 4 == 0 && host_aligned16(x_in) && host_aligned16(x_out) && host_aligned16(gain) && host_aligned16(n_out);
+      for (int t = 0; t < n_terms; ++t)
+        vec = vec && terms[t].y_row_stride % 4 == 0 && host_aligned16(terms[t].y) && host_aligned16(terms[t].bias) && host_aligned16(terms[t].norm_w);
       auto go = [&](auto npt) {
-        terms_rms_add_kernel<A, N, decltype(npt)::value><<<rows, 256, 0, as_stream(stream)>>>(
-            x_in, st_, x_out, static_cast<const A*>(gain), eps, static_cast<N*>(n_out), d);
+        if (vec)
+          terms_rms_add_kernel<A, N, decltype(npt)::value, true><<<rows, 256, 0, as_stream(stream)>>>(
+              x_in, st_, x_out, static_cast<const A*>(gain), eps, static_cast<N*>(n_out), d);
+        else
+          terms_rms_add_kernel<A, N, decltype(npt)::value, false><<<rows, 256, 0, as_stream(stream)>>>(
+              x_in, st_, x_out, static_cast<const A*>(gain), eps, static_cast<N*>(n_out), d);
       };
       if (d <= 1024) go(std::integral_constant<int, 4>());
       else if (d <= 4096) go(std::integral_constant<int, 16>());
