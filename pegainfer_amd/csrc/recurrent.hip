@@ -304,10 +304,9 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(const A* __restrict_
 // Selective state-space scan with a scalar decay per head (the state-space-duality form).  State per (slot, head): S [N][vdim].
 // xbc: fp32 rows [x: heads * vdim | B: groups * N | C: groups * N] (after their convolution and activation); the raw step sizes
 // come from the projection row (storage type), one per head.  B plays the key's part, C the query's, x the value's; no sum of a
-// token feeds the state, so four tokens' read-outs are in flight together.  COLS: value columns per workgroup, 16 (four waves) or
-// 8 (two waves) - the smaller form when heads x columns / 16 would leave compute units without a workgroup.
-template <int NS, typename A, int COLS>
-__global__ __launch_bounds__(COLS * 16) void ssd_scan_kernel(const float* __restrict__ xbc, int64_t xbc_stride, const A* __restrict__ proj,
+// token feeds the state, so four tokens' read-outs are in flight together.
+template <int NS, typename A>
+__global__ __launch_bounds__(256) void ssd_scan_kernel(const float* __restrict__ xbc, int64_t xbc_stride, const A* __restrict__ proj,
                                                        int64_t proj_stride, int64_t dt_off, const A* __restrict__ A_log,
                                                        const A* __restrict__ dt_bias, const A* __restrict__ Dskip,
                                                        float* __restrict__ state, int64_t slot_stride, float* __restrict__ o, int H,
@@ -316,7 +315,7 @@ __global__ __launch_bounds__(COLS * 16) void ssd_scan_kernel(const float* __rest
   constexpr int DP = kRecSlices * NS;
   __shared__ __attribute__((aligned(16))) float s_k[kRecTokens][DP], s_q[kRecTokens][DP];
   __shared__ float s_v[kRecTokens][kRecCols], s_a[kRecTokens], s_b[kRecTokens];
-  const int e = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * COLS;
+  const int e = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * kRecCols;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, cl = wave * 4 + (lane >> 4);
   const int col = col0 + cl;
   const int g0 = h / (H / G);
@@ -330,24 +329,19 @@ __global__ __launch_bounds__(COLS * 16) void ssd_scan_kernel(const float* __rest
   }
   const float rate = -expf(ld(A_log + h)), dtb = ld(dt_bias + h), skip = ld(Dskip + h);
   const int64_t b_at = (int64_t)H * vdim + (int64_t)g0 * dim, c_at = (int64_t)H * vdim + (int64_t)(G + g0) * dim;
-  // 16 threads stage a token; a workgroup of 8 columns has 128 threads and stages the round's tokens in two halves
-  constexpr int HALVES = 16 / COLS;
-  RoundFetch<NS> nxt[HALVES];
+  RoundFetch<NS> nxt;
   auto fetch = [&](int t0) {
     const float* base = xbc + (int64_t)(row0 + t0) * xbc_stride;
-#pragma unroll
-    for (int hv = 0; hv < HALVES; ++hv)
-      nxt[hv].issue(min(kRecTokens, len - t0), tid + hv * COLS * 16, dim,
-                    [=](int tt, int d) { return base[(int64_t)tt * xbc_stride + c_at + d]; },
-                    [=](int tt, int d) { return base[(int64_t)tt * xbc_stride + b_at + d]; },
-                    [=](int tt, int c) { return c < COLS && col0 + c < vdim ? base[(int64_t)tt * xbc_stride + (int64_t)h * vdim + col0 + c] : 0.f; });
+    nxt.issue(min(kRecTokens, len - t0), tid, dim,
+              [=](int tt, int d) { return base[(int64_t)tt * xbc_stride + c_at + d]; },
+              [=](int tt, int d) { return base[(int64_t)tt * xbc_stride + b_at + d]; },
+              [=](int tt, int c) { return col0 + c < vdim ? base[(int64_t)tt * xbc_stride + (int64_t)h * vdim + col0 + c] : 0.f; });
   };
   fetch(0);
   for (int t0 = 0; t0 < len; t0 += kRecTokens) {
     const int tc = min(kRecTokens, len - t0);
     __syncthreads();
-#pragma unroll
-    for (int hv = 0; hv < HALVES; ++hv) nxt[hv].land(tid + hv * COLS * 16, s_q, s_k, s_v);
+    nxt.land(tid, s_q, s_k, s_v);
     if (tid < kRecTokens) {   // rows past the entry's end: a = 1, b = 0 - a step that leaves S as it is
       const bool live = tid < tc;
       const float dt = live ? softplus_f(ld(proj + (int64_t)(row0 + t0 + tid) * proj_stride + dt_off + h) + dtb) : 0.f;
@@ -484,20 +478,15 @@ extern "C" pegainfer_status_t pegainfer_ssd_scan(const float* xbc, int64_t xbc_s
   if (n_entries <= 0) return 0;
   if (heads <= 0 || groups <= 0 || heads % groups || n_state <= 0 || n_state > 256 || vdim <= 0 || heads > 65535 || n_entries > 65535)
     return PK_BAD;
-  const bool narrow = vdim > 8 && (long)ceil_div(vdim, kRecCols) * heads * n_entries < device_cus();
-  const dim3 grid(ceil_div(vdim, narrow ? 8 : kRecCols), heads, n_entries);
+  const dim3 grid(ceil_div(vdim, kRecCols), heads, n_entries);
   bool ok = true;
   const bool known = by_dtype(dtype, [&](auto* t) {
     using A = std::remove_pointer_t<decltype(t)>;
     ok = by_slices(n_state, [&](auto ns) {
-      auto go = [&](auto kern, int threads) {
-        kern<<<grid, threads, 0, as_stream(stream)>>>(xbc, xbc_stride, static_cast<const A*>(proj), proj_stride, dt_off,
-                                                      static_cast<const A*>(A_log), static_cast<const A*>(dt_bias),
-                                                      static_cast<const A*>(D), state, slot_stride, o, heads, groups, n_state, vdim,
-                                                      entry_row0, entry_slot);
-      };
-      if (narrow) go(ssd_scan_kernel<decltype(ns)::value, A, 8>, 128);
-      else go(ssd_scan_kernel<decltype(ns)::value, A, 16>, 256);
+      ssd_scan_kernel<decltype(ns)::value, A><<<grid, 256, 0, as_stream(stream)>>>(
+          xbc, xbc_stride, static_cast<const A*>(proj), proj_stride, dt_off, static_cast<const A*>(A_log),
+          static_cast<const A*>(dt_bias), static_cast<const A*>(D), state, slot_stride, o, heads, groups, n_state, vdim, entry_row0,
+          entry_slot);
     });
   });
   return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
