@@ -187,6 +187,33 @@ def test_long_decoding_across_pages_key_tiles_and_window_edges():
     eng.close()
 
 
+def test_a_long_prompt_matches_its_portions_and_the_restatement():
+    """2100 tokens in one step (thirty key tiles, the window of 70 leaves most of them unvisited) against the same prompt in portions
+    and the restatement at some positions"""
+    cfg = C.config_tiny()
+    w = C.random_weights(cfg, 23)
+    toks = C.tokens_for(cfg, 2100, 9)
+    want = [0, 15, 16, 63, 64, 69, 70, 71, 72, 73, 500, 1023, 1024, 2047, 2048, 2099]
+    ref = C.oracle_logits(cfg, w, toks)[want]
+    for dtype in ("bfloat16", "float32"):
+        eng = C.engine_for(cfg, w, dtype, max_tokens=4400, max_requests=2)
+        a, b = eng.new_request(), eng.new_request()
+        whole = eng.step([(a, toks)], want=want)
+        check(whole, ref, dtype)
+        parts, at = [], 0
+        while at < len(toks):
+            n = min(150, len(toks) - at)
+            wn = [p - at for p in want if at <= p < at + n]
+            lg = eng.step([(b, toks[at:at + n])], want=wn)
+            if wn:
+                parts.append(lg)
+            at += n
+        got = np.concatenate(parts)
+        check(got, ref, dtype)
+        assert np.abs(whole - got).max() <= (1e-4 if dtype == "float32" else 0.1) * np.abs(whole).max()
+        eng.close()
+
+
 def test_graph_replays_of_decode_steps_match_eager_steps():
     """single-token steps are replayed from a captured graph: several replays, with prompt steps and synchronisations of other
     requests between them, against the same steps run eagerly (the per-layer tap switches the capture off)"""
