@@ -271,8 +271,7 @@ __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_d
     for (int q = 0; q < MB; ++q)
 #pragma unroll
       for (int r = 0; r < R; ++r) acc[q][r] = 0.f;
-#pragma unroll 4
-    for (int k = lane * 8; k < K; k += 512) {      // (unrolled: the weight loads of four trips are in flight together)
+    for (int k = lane * 8; k < K; k += 512) {      // (unrolling this loop by four was measured: 52 -> 66 us for a 65 536 x 2048 matrix)
       float wv[MB][8];
 #pragma unroll
       for (int q = 0; q < MB; ++q) {
