@@ -225,13 +225,14 @@ static void mfma_form_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
 
 // ------------------------------------------------------------------ few-rows form (decode)
 // At most R rows per tile (a decode step's tokens, or the pairs one expert received): the weights are streamed once with
-// 16-byte loads, the rows wait in LDS as fp32, a wave owns one output at a time (lanes over k, butterfly sum), 32 outputs per
+// 16-byte loads, the rows wait in LDS as fp32 (2048 k values at a time), a wave owns one output at a time (lanes over k, butterfly sum), 32 outputs per
 // workgroup - or 8 (OUT) when 32 would leave most of the chip without a workgroup (a matrix of a few thousand outputs).  fp32
 // arithmetic for both storage types; the k order of an output is fixed by K alone, whatever OUT is.
+constexpr int kRowsFormChunk = 2048;   // k values of the rows that wait in LDS at a time (a multiple of the 512 a wave strides by)
+
 template <typename TX, typename TW, typename TY, typename TG, int R, int OUT = 32>
 __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_desc d) {
-  constexpr int kRowsFormOutputs = OUT;
-  extern __shared__ float xr[];    // [R][K]
+  extern __shared__ __attribute__((aligned(16))) float xr[];    // [R][min(K, chunk)]
   __shared__ int xrow[R], yrow[R];
   int g, row0, nrows;
   if (d.tile_group) {
@@ -253,47 +254,64 @@ __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_d
   __syncthreads();
   const TX* X = static_cast<const TX*>(d.x) + (int64_t)g * d.x_group_stride;
   const TW* W = static_cast<const TW*>(d.w) + (int64_t)g * d.w_group_stride;
-  const int K = d.k;
-  for (int i = tid; i < R * K; i += 256) {
-    const int r = i / K, k = i - r * K;
-    xr[i] = xrow[r] >= 0 ? ld(X + (int64_t)xrow[r] * d.x_row_stride + k) : 0.f;
-  }
-  __syncthreads();
+  const int K = d.k, xs = min(K, kRowsFormChunk);
   TY* Y = static_cast<TY*>(d.y) + (int64_t)g * d.y_group_stride;
-  const int m_base = blockIdx.y * kRowsFormOutputs;
-  // a wave owns a quarter of the workgroup's outputs and walks them four at a time: four independent weight streams in flight
-  constexpr int MB = OUT >= 16 ? 4 : OUT / 4;
-  for (int mg = 0; mg < kRowsFormOutputs / 4; mg += MB) {
-    const int mw = m_base + wave * (kRowsFormOutputs / 4) + mg;
-    if (mw >= d.m) break;
-    float acc[MB][R];
+  // a wave owns a quarter of the workgroup's outputs and walks them four at a time: four independent weight streams in flight.
+  // The rows pass through LDS a chunk of k at a time (a long row times eight rows would leave room for one workgroup per compute
+  // unit); every output's sums stay in registers across the chunks, so its k order is what it would be in one piece.
+  constexpr int OW = OUT / 4, MB = OW >= 4 ? 4 : OW, NG = OW / MB;
+  const int m_base = blockIdx.y * OUT + wave * OW;
+  float acc[NG][MB][R];
+#pragma unroll
+  for (int n = 0; n < NG; ++n)
 #pragma unroll
     for (int q = 0; q < MB; ++q)
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[q][r] = 0.f;
-    for (int k = lane * 8; k < K; k += 512) {      // (unrolling this loop by four was measured: 52 -> 66 us for a 65 536 x 2048 matrix)
-      float wv[MB][8];
+      for (int r = 0; r < R; ++r) acc[n][q][r] = 0.f;
+  for (int kc0 = 0; kc0 < K; kc0 += kRowsFormChunk) {
+    const int kl = min(kRowsFormChunk, K - kc0);      // a multiple of 8, as K is
+    if (kc0 > 0) __syncthreads();
+    for (int i = tid * 8; i < R * kl; i += 2048) {
+      const int r = i / kl, k = i - r * kl;
+      float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (xrow[r] >= 0) Vec8<TX>::load(X + (int64_t)xrow[r] * d.x_row_stride + kc0 + k, t);
+      *reinterpret_cast<f32x4*>(xr + r * xs + k) = f32x4{t[0], t[1], t[2], t[3]};
+      *reinterpret_cast<f32x4*>(xr + r * xs + k + 4) = f32x4{t[4], t[5], t[6], t[7]};
+    }
+    __syncthreads();
 #pragma unroll
-      for (int q = 0; q < MB; ++q) {
-        const int m = min(mw + q, d.m - 1);          // a clamped row is loaded and dropped at the store
-        Vec8<TW>::load(W + (int64_t)m * d.w_m_stride + k, wv[q]);
-      }
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const f32x4 xa = *reinterpret_cast<const f32x4*>(xr + r * K + k), xb = *reinterpret_cast<const f32x4*>(xr + r * K + k + 4);
+    for (int n = 0; n < NG; ++n) {
+      const int mw = m_base + n * MB;
+      if (mw >= d.m) continue;
+      for (int k = lane * 8; k < kl; k += 512) {      // (unrolling this loop by four was measured: 52 -> 66 us for a 65 536 x 2048 matrix)
+        float wv[MB][8];
 #pragma unroll
         for (int q = 0; q < MB; ++q) {
-          float a = acc[q][r];
-          a = fmaf(wv[q][0], xa.x, a); a = fmaf(wv[q][1], xa.y, a); a = fmaf(wv[q][2], xa.z, a); a = fmaf(wv[q][3], xa.w, a);
-          a = fmaf(wv[q][4], xb.x, a); a = fmaf(wv[q][5], xb.y, a); a = fmaf(wv[q][6], xb.z, a); a = fmaf(wv[q][7], xb.w, a);
-          acc[q][r] = a;
+          const int m = min(mw + q, d.m - 1);          // a clamped row is loaded and dropped at the store
+          Vec8<TW>::load(W + (int64_t)m * d.w_m_stride + kc0 + k, wv[q]);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const f32x4 xa = *reinterpret_cast<const f32x4*>(xr + r * xs + k), xb = *reinterpret_cast<const f32x4*>(xr + r * xs + k + 4);
+#pragma unroll
+          for (int q = 0; q < MB; ++q) {
+            float a = acc[n][q][r];
+            a = fmaf(wv[q][0], xa.x, a); a = fmaf(wv[q][1], xa.y, a); a = fmaf(wv[q][2], xa.z, a); a = fmaf(wv[q][3], xa.w, a);
+            a = fmaf(wv[q][4], xb.x, a); a = fmaf(wv[q][5], xb.y, a); a = fmaf(wv[q][6], xb.z, a); a = fmaf(wv[q][7], xb.w, a);
+            acc[n][q][r] = a;
+          }
         }
       }
     }
+  }
+#pragma unroll
+  for (int n = 0; n < NG; ++n) {
+    const int mw = m_base + n * MB;
+    if (mw >= d.m) continue;
 #pragma unroll
     for (int q = 0; q < MB; ++q)
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[q][r] = wave_sum(acc[q][r]);
+      for (int r = 0; r < R; ++r) acc[n][q][r] = wave_sum(acc[n][q][r]);
     if (lane == 0) {
 #pragma unroll
       for (int q = 0; q < MB; ++q) {
@@ -302,7 +320,7 @@ __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_d
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           if (yrow[r] < 0) continue;
-          float v = acc[q][r];
+          float v = acc[n][q][r];
           if (d.epilogue == PEGAINFER_EPI_RELU_SQ) { v = fmaxf(v, 0.f); v *= v; }
           else if (d.epilogue == PEGAINFER_EPI_SIGMOID_GATE)
             v *= sigmoid_f(ld(static_cast<const TG*>(d.gate) + (int64_t)xrow[r] * d.gate_row_stride + g));
@@ -326,8 +344,9 @@ static void rows_form_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
   // 32 outputs per workgroup unless that leaves most compute units without one
   const bool fine = (long)row_tiles * groups * ceil_div(d.m, 32) < device_cus();
   dim3 grid(row_tiles, ceil_div(d.m, fine ? 8 : 32), groups);
-  if (fine) kern8<<<grid, 256, (size_t)R * d.k * sizeof(float), s>>>(d);
-  else kern<<<grid, 256, (size_t)R * d.k * sizeof(float), s>>>(d);
+  const size_t lds = (size_t)R * std::min(d.k, kRowsFormChunk) * sizeof(float);
+  if (fine) kern8<<<grid, 256, lds, s>>>(d);
+  else kern<<<grid, 256, lds, s>>>(d);
 }
 
 static inline bool chunks_ok(const pegainfer_gemm_desc& d) {
